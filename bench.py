@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the gfx950 filter-sparse conv2d path on one MI355X.
+
+A "step" is one pass of the hot path over one synthetic batch: every conv layer of the chosen suite
+(default: the VGG19-shaped stack at batch 16) launched once, back to back on one stream, inputs and
+packed weights already resident in HBM.  Prints ONE JSON line: whole-step dense-equivalent GFLOP/s
+(the reference's "FLOPS" figure, Tetris/spconv2d.cc:358, in decimal giga), per-layer microseconds and
+roofline fractions, the roofline of the conv kernel, and a CPU baseline measured on this box's cores.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--suite vgg19|resnet50|mobilenet|yolov3|single]
+                  [--batch N] [--no-cpu] [--no-check]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "tetris-artifact-evalution_amd"))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+
+PEAK_HBM_GBS = 8000.0        # MI355X published HBM3E bandwidth
+PEAK_FP32_TFLOPS = 157.3     # MI355X published vector/matrix fp32 peak
+
+# HBM bytes per step (all launches of spconv2d_kernel) from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# runs of this file, scaled by the same counters on a copy kernel of known size; see profiles/.  None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--suite", default="vgg19")
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
+    ap.add_argument("--layer-repeat", type=int, default=30, help="timed launches per layer for the per-layer table")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this engine runs on one GPU (no collectives or sharding are part of the path); "
+                 "--gpus %d is not supported" % args.gpus)
+
+    import numpy as np
+    import torch
+
+    import tetris_amd as T
+    from tetris_amd import workloads as W
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    layers = W.SUITES[args.suite]()
+    N = args.batch
+
+    packs, tiles, xs, ys, works = [], [], [], [], []
+    t_pack = 0.0
+    for L in layers:
+        w = W.make_weights(L)
+        tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+        t0 = time.perf_counter()
+        pk = T.G950Filter(w, tile.tile_ic)
+        torch.cuda.synchronize()
+        t_pack += time.perf_counter() - t0
+        x = torch.from_numpy(W.make_activations(L, N)).to(dev)
+        oh, ow = W.out_hw(L)
+        y = torch.empty((N, L.K, oh, ow), dtype=torch.float32, device=dev)
+        packs.append(pk); tiles.append(tile); xs.append(x); ys.append(y); works.append(W.work(L, N))
+    torch.cuda.synchronize()
+
+    def step():
+        for L, pk, tile, x, y in zip(layers, packs, tiles, xs, ys):
+            pk.launch(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # spot check of one mid-sized layer against the CPU oracle (not timed)
+    check = None
+    if not args.no_check:
+        import oracle_py as O
+        idx = min(range(len(layers)), key=lambda i: works[i]["flops_dense"] if layers[i].C > 3 else float("inf"))
+        L = layers[idx]
+        ref = O.host_conv2d(xs[idx][:1].cpu().numpy(), W.make_weights(L), L.stride, L.pad, threads=O.max_threads())
+        got = ys[idx][:1].cpu().numpy()
+        floor = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))  # same measure as tests/helpers.max_rel_err
+        err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+        check = {"layer": L.name, "max_rel_err": err, "tolerance": 1e-4, "ok": bool(err <= 1e-4)}
+
+    # per-layer table: events on the launch stream around back-to-back launches (reference protocol,
+    # Tetris/spconv2d.cc:44-68, with fewer repetitions so the default run stays short)
+    table = []
+    t_layers = 0.0
+    for L, pk, tile, x, y, wk in zip(layers, packs, tiles, xs, ys, works):
+        ms = pk.time(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile, warm=5, repeat=args.layer_repeat)
+        t = ms * 1e-3
+        t_layers += t
+        table.append({"layer": L.name, "us": round(ms * 1e3, 2),
+                      "gflops_dense_equiv": round(wk["flops_dense"] / t / 1e9, 1),
+                      "bound": wk["bound"], "roofline_frac": round(wk["t_roof"] / t, 4),
+                      "tile": [tile.lanes_w, tile.quads, tile.oc_per_wave, tile.waves, tile.tile_ic]})
+
+    fl_dense = sum(w["flops_dense"] for w in works)
+    fl_sparse = sum(w["flops_sparse"] for w in works)
+    bytes_alg = sum(w["bytes"] for w in works)
+    t_roof = sum(w["t_roof"] for w in works)
+    n_launch = len(layers)
+    t_hbm, t_fp32 = bytes_alg / (PEAK_HBM_GBS * 1e9), fl_sparse / (PEAK_FP32_TFLOPS * 1e12)
+    if t_fp32 >= t_hbm:
+        achieved = fl_sparse / t_layers / 1e12
+        roofline = {"bound": "mfma", "bound_detail": "vector fp32 FMA issued from the VALU; no MFMA is used. Peak is the "
+                    "published 157.3 TFLOP/s fp32 figure, which needs packed fp32 FMA; this build compiles with packed "
+                    "fp32 off, so 78.6 TFLOP/s is the most its instructions can reach",
+                    "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_FP32_TFLOPS, 4)}
+    else:
+        achieved = bytes_alg / t_layers / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    roofline.update({"kernel": "spconv2d_kernel", "launches_per_step": n_launch,
+                     "avg_launch_us": round(t_layers / n_launch * 1e6, 2),
+                     "algorithmic_flops_per_launch": fl_sparse / n_launch,
+                     "algorithmic_bytes_per_launch": bytes_alg / n_launch,
+                     "sum_of_layer_roofs_frac": round(t_roof / t_layers, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("%s/%d" % (args.suite, N))})
+
+    cpu = None
+    if not args.no_cpu:
+        import oracle_py as O
+        threads = min(O.max_threads(), 16)
+        sample_layers = W.SUITES[args.suite]()
+        budget_s, done_fl, t_cpu, used = 20.0, 0.0, 0.0, 0
+        for L in sample_layers:
+            w = W.make_weights(L)
+            x1 = W.make_activations(L, 1)
+            pk = O.G950Pack(w, 32)
+            t0 = time.perf_counter()
+            pk.conv(x1, L.stride, L.pad, threads=threads)
+            t_cpu += time.perf_counter() - t0
+            done_fl += W.work(L, 1)["flops_dense"]
+            used += 1
+            if t_cpu > budget_s:
+                break
+        cpu = {"value": round(done_fl / t_cpu / 1e9, 2), "unit": "GFLOP/s (dense-equiv)", "cores": threads,
+               "kind": "port", "sample": "first %d of %d %s layers at batch 1, packed-format decode conv of the oracle "
+               "(restates HostReorderSpconv2d, spconv2d_utils.h:457-493), OpenMP over (n, oc), %.1f s" % (
+                   used, len(sample_layers), args.suite, t_cpu)}
+        if O.ref_available():
+            L = W.single_layer()[0]
+            w, x1 = W.make_weights(L), W.make_activations(L, 1)
+            t0 = time.perf_counter()
+            O.ref_host_conv2d(x1, w, L.stride, L.pad)
+            dt = time.perf_counter() - t0
+            cpu["reference_HostConv2d"] = {"value": round(W.work(L, 1)["flops_dense"] / dt / 1e9, 3),
+                                           "unit": "GFLOP/s (dense-equiv)", "cores": 1, "kind": "reference",
+                                           "sample": "single 64->128 56x56 3x3 layer, batch 1, %.2f s" % dt}
+
+    out = {
+        "metric": "effective GFLOP/s (dense-equivalent) over the layer stack; per-layer us and roofline in `layers`",
+        "value": round(fl_dense / (ms_per_step * 1e-3) / 1e9, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s-shaped sparse conv stack, %d layers, batch %d, fp32 NCHW, seeded unstructured masks"
+                   % (args.suite, len(layers), N), "suite": args.suite, "batch": N, "layers": len(layers)},
+        "sparse_gflops": round(fl_sparse / (ms_per_step * 1e-3) / 1e9, 1),
+        "sum_layer_us": round(t_layers * 1e6, 1),
+        "pack_ms_total": round(t_pack * 1e3, 2),
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "check": check,
+        "layers": table,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

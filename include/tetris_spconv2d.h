@@ -1,0 +1,164 @@
+/* C ABI of the MI355X (gfx950) filter-sparse conv2d engine.
+ *
+ * Every entry point replaces one interface of the reference's spconv2d / spf path (file:line are
+ * relative to the reference checkout).  Pointers named h_* are host memory, d_* device memory of the
+ * current HIP device.  All tensors are fp32; indices are int32.  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  Every function returns 0 on success or a TETRIS_E* code;
+ * tetris_last_error() gives the message of the calling thread's last failure.  Nothing here exits
+ * the process (the reference's checkCudaErrors prints and calls exit, Tetris/cuda_utils.h:9-16).
+ */
+#ifndef TETRIS_SPCONV2D_H_
+#define TETRIS_SPCONV2D_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  TETRIS_OK = 0,
+  TETRIS_EINVAL = 1,      /* bad argument (shape, NULL, ks > 7, ...) */
+  TETRIS_EHIP = 2,        /* a HIP call failed */
+  TETRIS_EUNSUPPORTED = 3,/* reference behaviour undefined for this input (see tetris_spf_create) */
+  TETRIS_ENOTFOUND = 4,   /* raw device arrays not produced by a live tetris_spf handle */
+  TETRIS_EIO = 5          /* weight file cannot be opened or is truncated */
+};
+
+/* The reference's two compile-time packer macros (Tetris/spconv2d_utils.h:66, :80), as run-time flags. */
+#define TETRIS_BANK_OPTIMIZE 1u
+#define TETRIS_REORDER_OUT_CHANNEL 2u
+
+const char* tetris_last_error(void);
+const char* tetris_version(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * Weight preprocessing, reference layout ("SPF").
+ * Replaces: struct SparseFilter<float,int,int> -- constructor Tetris/spconv2d_utils.h:25-265,
+ * destructor :267-273, getters :495-500, public vectors :505-509.
+ * The five arrays are byte-identical to the reference's for the same arguments and macro set.
+ * TETRIS_EUNSUPPORTED is returned when Bank-SR would read its 32 bank flags out of range
+ * (spconv2d_utils.h:184 indexes them by an entry index), where the reference's result is undefined.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct tetris_spf tetris_spf;
+
+int tetris_spf_create(const float* h_filter_oihw, int in_channel, int out_channel, int kernel_size, int tile_ic,
+                      int apply_reorder, int apply_vectorize, unsigned flags, tetris_spf** out);
+void tetris_spf_destroy(tetris_spf* f);
+
+typedef struct tetris_spf_arrays {
+  const int32_t* offsets;        int64_t n_offsets;         /* offsets_         */
+  const int32_t* stage_len;      int64_t n_stage_len;       /* stage_len_       */
+  const int32_t* position;       int64_t n_position;        /* position_        */
+  const float*   values;         int64_t n_values;          /* values_          */
+  const int32_t* oc_permutation; int64_t n_oc_permutation;  /* oc_permutation_  */
+  int64_t nnz;                   /* nnz_ (counted on the apply_reorder == 0 path only, like the reference) */
+  int32_t tile_ic;               /* GetTileIC() */
+} tetris_spf_arrays;
+
+int tetris_spf_host_arrays(const tetris_spf* f, tetris_spf_arrays* out);   /* the public vectors */
+/* GetDevice*(): the device copies are made on the first call (the reference uploads in its constructor). */
+int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Weight preprocessing, gfx950 layout: a device pass (count, scan, scatter) over the dense OIHW
+ * filter that writes, per (output-channel slot, input-channel stage), the non-zero entries in
+ * (channel, row, column) order, padded with zero entries to a multiple of 8 so that a wave fetches
+ * eight (offset, value) pairs with one 64-byte scalar load.
+ * No reference counterpart for the layout; it plays the role of the SparseFilter constructor for the
+ * HIP kernel.  `oc_order` (may be NULL = identity) lists, slot by slot, which output channel a slot
+ * computes -- pass a tetris_spf's oc_permutation to keep the reference's channel regrouping.
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct tetris_g950 tetris_g950;
+
+int tetris_g950_create(const float* h_filter_oihw, int in_channel, int out_channel, int kernel_size, int tile_ic,
+                       const int32_t* oc_order, void* stream, tetris_g950** out);
+/* Same, from a filter already resident in device memory. */
+int tetris_g950_create_device(const float* d_filter_oihw, int in_channel, int out_channel, int kernel_size,
+                              int tile_ic, const int32_t* oc_order, void* stream, tetris_g950** out);
+void tetris_g950_destroy(tetris_g950* p);
+
+typedef struct tetris_g950_arrays {
+  const int32_t* seg_offsets; int64_t n_seg_offsets; /* [slots*stages+1], entry index, multiples of 8 */
+  const int32_t* seg_nnz;     int64_t n_seg_nnz;     /* [slots*stages], real entries in the segment    */
+  const int32_t* position;    int64_t n_entries;     /* s | r<<3 | (ic % tile_ic)<<6, 0 for padding    */
+  const float*   values;                             /* 0.0f for padding                               */
+  const int32_t* oc_order;    int64_t n_slots;       /* output channel of each slot                    */
+  int32_t stages, tile_ic;
+  int64_t nnz;
+} tetris_g950_arrays;
+
+/* Copies the packed arrays to host memory owned by the handle (valid until it is destroyed). */
+int tetris_g950_host_arrays(tetris_g950* p, tetris_g950_arrays* out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Tile shape of the conv kernel.  Replaces the template arguments <TILE_IC, TILE_H, TILE_W> of the
+ * reference launcher and its exhaustive table (Tetris/spconv2d.cc:90-329).  A zeroed struct means
+ * "choose for me".
+ * ---------------------------------------------------------------------------------------------- */
+typedef struct tetris_tile {
+  int32_t lanes_w;     /* lanes across a tile row; the tile is 4*lanes_w output columns wide      */
+  int32_t quads;       /* 4-pixel groups per lane (1, 2 or 4)                                      */
+  int32_t oc_per_wave; /* output channels a wave accumulates at once (4, 8 or 16)                  */
+  int32_t waves;       /* waves per workgroup (1..16); workgroup computes waves*oc_per_wave channels */
+  int32_t tile_ic;     /* input channels staged in LDS at a time (informative on launch: the pack's) */
+} tetris_tile;
+
+int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_channel, int kernel_size, int stride,
+                       int padding, tetris_tile* out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Conv launch on device tensors.  Replaces: SparseConv2d<float,int,int,KS,STRIDE,TILE_IC,TILE_H,TILE_W>
+ * (Tetris/spconv2d_kernel.cuh:14-21, Tetris/spconv2d_kernel.cu:163-188).  Asynchronous on `stream`.
+ * d_input is NCHW [batch][in_channel][img_h][img_w], d_output NCHW [batch][out_channel][oh][ow] with
+ * oh = (img_h + 2*padding - kernel_size)/stride + 1 (the reference keeps NHWC on the device; its host
+ * entry points below take and return NCHW, as here).
+ * ---------------------------------------------------------------------------------------------- */
+int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
+                           int stride, int padding, const tetris_tile* tile, void* stream);
+
+/* Same call shape as the reference launcher: the raw device arrays of a live tetris_spf (looked up by
+ * `d_values`).  tile_h/tile_w are accepted for source compatibility and ignored. */
+int tetris_spconv2d_launch_spf(const float* d_input, const int32_t* d_offsets, const int32_t* d_stage_len,
+                               const int32_t* d_oc_permutation, const int32_t* d_position, const float* d_values,
+                               float* d_output, int batch, int img_h, int img_w, int in_channel, int out_channel,
+                               int kernel_size, int stride, int padding, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Host-to-host entry points.
+ * tetris_spconv2d_host  replaces CudaSparseConv2d<float,int,int>  (Tetris/spconv2d.cc:332-367)
+ * tetris_spconv2d_spf_host replaces SparseConv2d_SPF<float,int,int> (Tetris/spf.cc:22-93)
+ * h_input NCHW, h_filter OIHW, h_output NCHW.  Both upload, pack, time the launch with the reference's
+ * protocol (30 warm-up + 100 timed launches between two events, Tetris/tensor_utils.h:10-11), and
+ * download.  *ms_out (may be NULL) receives the mean milliseconds per launch.  `layout` is accepted
+ * for source compatibility ("NHWC" in the reference's mains) and does not change the host layout.
+ * ---------------------------------------------------------------------------------------------- */
+int tetris_spconv2d_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
+                         int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
+                         void* stream, const char* layout, int apply_reorder, float* ms_out);
+int tetris_spconv2d_spf_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
+                             int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
+                             void* stream, const char* layout, int apply_reorder, float* ms_out);
+
+/* Times `repeat` back-to-back launches after `warm` untimed ones (TimingTetrisSparseConv2d,
+ * Tetris/spconv2d.cc:29-69); mean milliseconds per launch in *ms_out. */
+int tetris_spconv2d_time(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
+                         int stride, int padding, const tetris_tile* tile, void* stream, int warm, int repeat,
+                         float* ms_out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Utilities of the path.
+ * tetris_read_weight_file replaces ReadConfigAndDataFromFile (Tetris/tensor_utils.cc:55-82); header
+ * order H W IC OC KS PAD STRIDE GROUPS; *h_filter_out is malloc'ed, release with tetris_free.
+ * tetris_float_equal / tetris_tensor_equal replace FloatEqual / TensorEqual (:17-34).
+ * ---------------------------------------------------------------------------------------------- */
+int tetris_read_weight_file(const char* path, int32_t header[8], float** h_filter_out, int64_t* nnz_out);
+void tetris_free(void* p);
+int tetris_float_equal(float x, float y);
+int64_t tetris_tensor_first_mismatch(const float* x, const float* y, int64_t len); /* -1 when equal */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TETRIS_SPCONV2D_H_ */

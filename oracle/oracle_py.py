@@ -58,6 +58,15 @@ if _lib is not None:
         getattr(_lib, "orc_pack_" + _n).restype = C.POINTER(_t)
     _lib.orc_host_spconv2d.argtypes = [C.c_void_p, _f32p, _f32p] + [C.c_int] * 6
     _lib.orc_host_reorder_spconv2d.argtypes = [C.c_void_p, _f32p, _f32p] + [C.c_int] * 6
+    _lib.orc_g950_pack.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    _lib.orc_g950_pack.restype = C.c_void_p
+    _lib.orc_g950_free.argtypes = [C.c_void_p]
+    _lib.orc_g950_sizes.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
+    for _n, _t in (("seg_off", C.c_int32), ("seg_nnz", C.c_int32), ("position", C.c_int32), ("values", C.c_float),
+                   ("order", C.c_int32)):
+        getattr(_lib, "orc_g950_" + _n).argtypes = [C.c_void_p]
+        getattr(_lib, "orc_g950_" + _n).restype = C.POINTER(_t)
+    _lib.orc_g950_conv.argtypes = [C.c_void_p, _f32p, _f32p] + [C.c_int] * 6
     _lib.orc_fnv1a.argtypes = [C.c_void_p, C.c_int64, C.c_uint64]
     _lib.orc_fnv1a.restype = C.c_uint64
     _lib.orc_max_threads.restype = C.c_int
@@ -184,8 +193,48 @@ class SpfPack:
         return out
 
     def __del__(self):
-        if getattr(self, "_h", None):
+        if getattr(self, "_h", None) and _lib is not None:
             _lib.orc_pack_free(self._h)
+            self._h = None
+
+
+class G950Pack:
+    """Result of orc_g950_pack: the layout the HIP kernel consumes, built on the CPU."""
+
+    def __init__(self, w, tile_ic, order=None):
+        w = np.ascontiguousarray(w, np.float32)
+        self.K, self.C, self.ks, _ = w.shape
+        self.tile_ic = tile_ic
+        o = None if order is None else np.ascontiguousarray(order, np.int32)
+        self._h = _lib.orc_g950_pack(w, self.C, self.K, self.ks, tile_ic,
+                                     None if o is None else o.ctypes.data_as(C.c_void_p))
+        n = (C.c_int64 * 5)()
+        _lib.orc_g950_sizes(self._h, n)
+        self.slots, self.stages = int(n[3]), int(n[4])
+
+        def grab(name, cnt, dt):
+            if cnt == 0:
+                return np.zeros(0, dt)
+            return np.ctypeslib.as_array(getattr(_lib, "orc_g950_" + name)(self._h), shape=(cnt,)).copy()
+
+        self.seg_off = grab("seg_off", n[0], np.int32)
+        self.seg_nnz = grab("seg_nnz", n[1], np.int32)
+        self.position = grab("position", n[2], np.int32)
+        self.values = grab("values", n[2], np.float32)
+        self.order = grab("order", n[3], np.int32)
+
+    def conv(self, x, stride, pad, threads=1):
+        x = np.ascontiguousarray(x, np.float32)
+        n, c, h, wd = x.shape
+        assert c == self.C
+        out = np.zeros((n, self.K, out_extent(h, pad, self.ks, stride), out_extent(wd, pad, self.ks, stride)),
+                       np.float32)
+        _lib.orc_g950_conv(self._h, x, out, n, h, wd, pad, stride, threads)
+        return out
+
+    def __del__(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.orc_g950_free(self._h)
             self._h = None
 
 

@@ -497,6 +497,89 @@ void orc_host_reorder_spconv2d(const OrcPack* p, const float* input, float* outp
         }
 }
 
+// ---- gfx950 layout (defined by this project; no reference counterpart) --------------------------
+// Slots = K rounded up to a multiple of 128; slot i computes output channel order[i] (identity when
+// order == NULL), padding slots hold -1 and empty runs.  Per (slot, stage): the non-zero weights of
+// channels [stage*tile_ic, ...) in (channel, row, column) order -- the scan order of
+// spconv2d_utils.h:85-94 -- with the reference's position word (:91), then (0, 0.0f) entries up to a
+// multiple of 8.  seg_off is the running sum of the padded run lengths.
+struct OrcG950 {
+  int C = 0, K = 0, ks = 0, tile_ic = 0, stages = 0, slots = 0;
+  std::vector<int32_t> seg_off, seg_nnz, position, order;
+  std::vector<float> values;
+};
+
+OrcG950* orc_g950_pack(const float* filter, int C, int K, int ks, int tile_ic, const int32_t* order) {
+  OrcG950* P = new OrcG950;
+  P->C = C; P->K = K; P->ks = ks; P->tile_ic = tile_ic;
+  P->stages = (C - 1) / tile_ic + 1;
+  P->slots = (K + 127) / 128 * 128;
+  P->order.assign(P->slots, -1);
+  for (int i = 0; i < K; ++i) P->order[i] = order ? order[i] : i;
+  P->seg_off.push_back(0);
+  const int kk = ks * ks;
+  for (int slot = 0; slot < P->slots; ++slot)
+    for (int st = 0; st < P->stages; ++st) {
+      int n = 0;
+      const int oc = P->order[slot];
+      if (oc >= 0)
+        for (int j = st * tile_ic; j < std::min((st + 1) * tile_ic, C); ++j)
+          for (int r = 0; r < ks; ++r)
+            for (int s = 0; s < ks; ++s) {
+              const float v = filter[(size_t)oc * C * kk + (size_t)j * kk + r * ks + s];
+              if (v != 0.f) {
+                P->position.push_back(make_pos(s, r, j % tile_ic));
+                P->values.push_back(v);
+                ++n;
+              }
+            }
+      P->seg_nnz.push_back(n);
+      for (int i = n; i % 8 != 0; ++i) {
+        P->position.push_back(0);
+        P->values.push_back(0.0f);
+      }
+      P->seg_off.push_back((int32_t)P->position.size());
+    }
+  return P;
+}
+void orc_g950_free(OrcG950* p) { delete p; }
+void orc_g950_sizes(const OrcG950* p, int64_t* n) {
+  n[0] = (int64_t)p->seg_off.size(); n[1] = (int64_t)p->seg_nnz.size(); n[2] = (int64_t)p->position.size();
+  n[3] = p->slots; n[4] = p->stages;
+}
+const int32_t* orc_g950_seg_off(const OrcG950* p) { return p->seg_off.data(); }
+const int32_t* orc_g950_seg_nnz(const OrcG950* p) { return p->seg_nnz.data(); }
+const int32_t* orc_g950_position(const OrcG950* p) { return p->position.data(); }
+const float* orc_g950_values(const OrcG950* p) { return p->values.data(); }
+const int32_t* orc_g950_order(const OrcG950* p) { return p->order.data(); }
+
+// Convolution straight from the gfx950 arrays, accumulating in run order (stage by stage, entry by
+// entry, padding entries included) -- the order the HIP kernel adds in, without its fused multiply-add.
+void orc_g950_conv(const OrcG950* p, const float* input, float* output, int N, int H, int W, int pad, int stride,
+                   int threads) {
+  const int C = p->C, K = p->K, ks = p->ks, S = p->stages, T = p->tile_ic;
+  const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
+#pragma omp parallel for collapse(2) schedule(dynamic) num_threads(threads > 0 ? threads : 1)
+  for (int n = 0; n < N; ++n)
+    for (int slot = 0; slot < p->slots; ++slot) {
+      const int oc = p->order[slot];
+      if (oc < 0) continue;
+      for (int h = 0; h < OH; ++h)
+        for (int w = 0; w < OW; ++w) {
+          float sum = 0;
+          for (int st = 0; st < S; ++st)
+            for (int e = p->seg_off[slot * S + st]; e < p->seg_off[slot * S + st + 1]; ++e) {
+              const int pos = p->position[e];
+              const int y = pos & 7, x = (pos >> kBitS) & 7, ic = (pos >> (kBitS + kBitR)) + st * T;
+              const int ih = h * stride + x, iw = w * stride + y;
+              if (ih < pad || ih >= H + pad || iw < pad || iw >= W + pad) continue;
+              sum += input[(((size_t)n * C + ic) * H + (ih - pad)) * W + (iw - pad)] * p->values[e];
+            }
+          output[(((size_t)n * K + oc) * OH + h) * OW + w] = sum;
+        }
+    }
+}
+
 // FNV-1a 64 over raw bytes; pass the previous return value as `h` to chain buffers
 // (the known-answer table starts from 1469598103934665603, see oracle_py.py).
 uint64_t orc_fnv1a(const void* data, int64_t len, uint64_t h) {

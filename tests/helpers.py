@@ -19,8 +19,17 @@ def relu_like(rng, shape):
     return x
 
 
-def max_rel_err(got, ref, eps=1e-3):
-    """max |got-ref| / max(|ref|, eps): the denominator floor keeps exact-zero outputs meaningful."""
+def max_rel_err(got, ref, eps=None):
+    """max |got-ref| / max(|ref|, eps) with eps = max(1e-3, 1% of the largest |ref|).
+
+    The floor is needed because ReLU-like inputs and cancelling sums give outputs at or near zero, where two
+    correct fp32 summation orders differ by a few 1e-8 absolute; tying it to the tensor's scale keeps the bar
+    at 1e-6 of the largest output.  (The reference's own predicate allows 1e-5 absolute, tensor_utils.cc:17-19.)
+    """
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
-    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps))) if ref.size else 0.0
+    if not ref.size:
+        return 0.0
+    if eps is None:
+        eps = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))
+    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), eps)))

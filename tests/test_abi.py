@@ -1,0 +1,94 @@
+"""CPU-side checks of the shipped library: it loads, exports what include/tetris_spconv2d.h declares,
+rejects bad arguments with a message, and its host packer equals the oracle byte for byte."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from conftest import GOLDEN, ROOT, golden_weights
+from helpers import sparse_filter
+
+T = pytest.importorskip("tetris_amd")
+
+
+def test_every_declared_symbol_is_exported():
+    hdr = open(os.path.join(ROOT, "include", "tetris_spconv2d.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    names = set(re.findall(r"\b(tetris_[a-z0-9_]+)\s*\(", hdr))
+    assert len(names) >= 20
+    lib = ctypes.CDLL(T.LIB_PATH)
+    missing = [n for n in sorted(names) if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_version_and_errors():
+    assert "gfx950" in T.version()
+    w = np.zeros((4, 4, 9, 9), np.float32)
+    with pytest.raises(T.TetrisError) as e:
+        T.SparseFilter(w, 4, 4, 9)  # 3-bit row/column fields: kernel_size <= 7
+    assert e.value.code == T.EINVAL and "ks" in str(e.value)
+    with pytest.raises(T.TetrisError) as e:
+        T.ReadConfigAndDataFromFile("/nonexistent/weights")
+    assert e.value.code == T.EIO and "Open file error" in str(e.value)
+
+
+CASES = [(40, 20, 3, 8, 0.8), (64, 48, 1, 32, 0.7), (33, 7, 3, 32, 0.5), (70, 70, 1, 32, 0.9), (16, 3, 7, 32, 0.85),
+         (96, 40, 3, 16, 0.95), (8, 64, 3, 64, 0.9), (255, 64, 1, 128, 0.75)]
+MODES = [(0, 1, 0), (1, 0, 0), (1, 1, 0), (1, 1, T.BANK_OPTIMIZE), (1, 1, T.REORDER_OUT_CHANNEL),
+         (1, 1, T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL), (1, 0, T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL)]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_sparse_filter_equals_oracle_bytes(oracle, case):
+    K, C, ks, tic, sp = case
+    w = sparse_filter(np.random.default_rng(K * 1000 + C + ks), K, C, ks, sp)
+    for reorder, vec, flags in MODES:
+        o = oracle.SpfPack(w, tic, bool(reorder), bool(vec), bool(flags & 1), bool(flags & 2))
+        assert o.bank_oob == 0
+        p = T.SparseFilter(w, C, K, ks, tic, bool(reorder), bool(vec), flags)
+        for a, b in zip(o.arrays(), p.arrays()):
+            assert a.dtype == b.dtype and a.tobytes() == b.tobytes()
+        assert p.nnz_ == o.nnz_counted and p.GetTileIC() == tic
+        p.close()
+
+
+@pytest.mark.parametrize("name", ["rn90_3x3", "rn90_stem", "rn98_1x1", "vgg_64x128", "yolo_255"])
+def test_sparse_filter_on_shipped_layers(oracle, name):
+    import json
+    rows = [r for r in json.load(open(os.path.join(GOLDEN, "spf_known_answers.json")))["rows"] if r["layer"] == name]
+    hdr, w, _ = golden_weights(name)
+    for r in rows:
+        flags = (T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL) if r["flags"] == "BR" else 0
+        p = T.SparseFilter(w, hdr["IC"], hdr["OC"], hdr["KS"], r["tile_ic"], True, True, flags)
+        assert "%016x" % oracle.fnv1a(*p.arrays()) == r["fnv_all"]
+        assert "%016x" % oracle.fnv1a(p.oc_permutation_) == r["fnv_perm"]
+        p.close()
+
+
+def test_reader_and_tolerance_match_oracle(oracle, tmp_path):
+    vals = np.array([0.0, -0.0, 1.5, -2.25e-3, 7, 1e-8, 0.0, 3.25], np.float32)
+    p = tmp_path / "w.txt"
+    p.write_text("5 6 2 4 1 0 1 1\n" + " ".join(repr(float(v)) for v in vals) + "\n")
+    hdr, w, nnz = T.ReadConfigAndDataFromFile(str(p))
+    hdr_o, w_o, nnz_o = oracle.read_weight_file(str(p))
+    assert hdr == hdr_o and nnz == nnz_o == 5 and w.tobytes() == w_o.tobytes()
+    (tmp_path / "short.txt").write_text("5 6 2 4 1 0 1 1\n0.5 0.25\n")
+    with pytest.raises(T.TetrisError) as e:
+        T.ReadConfigAndDataFromFile(str(tmp_path / "short.txt"))
+    assert e.value.code == T.EIO
+    for a, b in [(0.0, 1e-5), (0.0, 1.01e-5), (1.0, 1.00003), (1.0, 1.00002), (1e6, 1e6 + 25), (1.0, -1.0)]:
+        assert T.FloatEqual(a, b) == oracle.float_equal(a, b)
+    x = np.arange(8, dtype=np.float32)
+    assert T.TensorEqual(x, x.copy()) and not T.TensorEqual(x, x + 1)
+
+
+def test_tile_select_is_sane():
+    for shape in [(1, 56, 56, 64, 128, 3, 1, 1), (16, 224, 224, 3, 64, 3, 1, 1), (16, 7, 7, 1024, 1024, 1, 1, 0),
+                  (4, 224, 224, 3, 64, 7, 2, 3), (16, 13, 13, 1024, 255, 1, 1, 0), (1, 14, 14, 512, 512, 3, 1, 1)]:
+        t = T.tile_select(*shape)
+        assert 1 <= t.lanes_w <= 16 and t.quads in (1, 2, 4) and t.oc_per_wave in (4, 8, 16)
+        assert t.waves in (1, 2, 4, 8) and t.tile_ic >= 1
+    with pytest.raises(T.TetrisError):
+        T.tile_select(0, 5, 5, 3, 3, 3, 1, 1)

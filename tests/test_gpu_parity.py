@@ -1,0 +1,212 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle, on a real MI355X.
+
+Bars: packed index arrays bit-exact; fp32 outputs within max relative error 1e-4, measured as
+max |got-ref| / max(|ref|, eps), eps = max(1e-3, 1% of the largest |ref|) (see helpers.max_rel_err).
+"""
+import os
+
+import numpy as np
+import pytest
+
+from conftest import REFERENCE, golden_weights
+from helpers import max_rel_err, relu_like, sparse_filter
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.fixture(scope="module")
+def env(oracle):
+    import torch
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import tetris_amd as T
+
+    return T, torch, oracle
+
+
+def run_conv(T, torch, pk, x, K, ks, stride, pad, tile=None):
+    n, c, h, w = x.shape
+    dx = torch.from_numpy(x).cuda()
+    dy = torch.full((n, K, T.out_extent(h, pad, ks, stride), T.out_extent(w, pad, ks, stride)), float("nan"),
+                    device="cuda")
+    pk.launch(dx.data_ptr(), dy.data_ptr(), n, h, w, stride, pad, tile)
+    torch.cuda.synchronize()
+    return dy.cpu().numpy()
+
+
+SHAPES = [  # N, C, H, W, K, ks, stride, pad, sparsity  -- the reference's kernel-size/stride families, ragged edges
+    (1, 8, 12, 12, 16, 3, 1, 1, 0.7),
+    (2, 20, 9, 11, 40, 3, 1, 1, 0.8),
+    (1, 48, 8, 8, 64, 1, 1, 0, 0.7),
+    (1, 7, 13, 13, 33, 3, 2, 1, 0.5),
+    (2, 3, 17, 17, 16, 7, 2, 3, 0.85),
+    (1, 70, 6, 6, 70, 1, 2, 0, 0.9),
+    (3, 16, 14, 14, 32, 3, 1, 1, 0.9),
+    (5, 32, 7, 7, 64, 1, 1, 0, 0.8),
+    (1, 130, 5, 9, 129, 3, 1, 0, 0.9),
+    (2, 4, 30, 61, 8, 5, 1, 2, 0.6),
+    (1, 16, 10, 10, 24, 3, 1, 1, 1.0),   # all-zero filter
+    (1, 16, 10, 10, 24, 3, 1, 1, 0.0),   # dense filter
+    (17, 5, 3, 3, 260, 1, 1, 0, 0.5),    # more images than a tile folds, K over two slot paddings
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_conv_matches_oracle(env, shape):
+    T, torch, O = env
+    N, C, H, W, K, ks, stride, pad, sp = shape
+    rng = np.random.default_rng(sum(shape[:8]))
+    w = sparse_filter(rng, K, C, ks, sp)
+    x = relu_like(rng, (N, C, H, W))
+    tile = T.tile_select(N, H, W, C, K, ks, stride, pad)
+    pk = T.G950Filter(w, tile.tile_ic)
+    a, o = pk.host_arrays(), O.G950Pack(w, tile.tile_ic)
+    assert np.array_equal(a["seg_offsets"], o.seg_off) and np.array_equal(a["seg_nnz"], o.seg_nnz)
+    assert np.array_equal(a["position"], o.position) and a["values"].tobytes() == o.values.tobytes()
+    assert np.array_equal(a["oc_order"], o.order) and a["nnz"] == int((w != 0).sum())
+    y = run_conv(T, torch, pk, x, K, ks, stride, pad, tile)
+    assert not np.isnan(y).any()
+    ref = O.host_conv2d(x, w, stride, pad, threads=4)
+    assert max_rel_err(y, ref) <= TOL
+    # same arrays decoded on the CPU in the same accumulation order
+    assert max_rel_err(y, o.conv(x, stride, pad, threads=4)) <= TOL
+    assert T.TensorEqual(y, ref)  # the reference's own predicate (tensor_utils.cc:17-34)
+
+
+TILES = [(16, 2, 8, 4), (8, 2, 8, 4), (4, 2, 8, 2), (2, 2, 8, 4), (14, 2, 8, 4), (7, 2, 8, 8), (13, 1, 16, 4),
+         (16, 4, 8, 4), (8, 4, 4, 8), (16, 1, 8, 1), (4, 2, 16, 8), (1, 2, 4, 4), (16, 2, 4, 4), (5, 4, 8, 2)]
+
+
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("conv", [(3, 1, 1), (1, 1, 0), (3, 2, 1), (7, 2, 3), (1, 2, 0)])
+def test_every_tile_shape(env, tile, conv):
+    T, torch, O = env
+    ks, stride, pad = conv
+    lw, nq, g, waves = tile
+    N, C, H, W, K = 3, 12, 23, 29, 37
+    rng = np.random.default_rng(lw * 100 + nq * 10 + g + ks + stride)
+    w = sparse_filter(rng, K, C, ks, 0.7)
+    x = relu_like(rng, (N, C, H, W))
+    ref = O.host_conv2d(x, w, stride, pad, threads=4)
+    ran = 0
+    for tile_ic in (2, 5, 16):
+        t = T.Tile(lw, nq, g, waves, tile_ic)
+        pk = T.G950Filter(w, tile_ic)
+        try:
+            y = run_conv(T, torch, pk, x, K, ks, stride, pad, t)
+        except T.TetrisError as e:  # the biggest tiles do not fit 160 KB of LDS with 16 staged channels
+            assert e.code == T.EINVAL and "LDS" in str(e) and tile_ic > 2
+            continue
+        ran += 1
+        assert max_rel_err(y, ref) <= TOL, (tile, conv, tile_ic)
+    assert ran >= 1
+
+
+def test_channel_order_is_honoured(env):
+    T, torch, O = env
+    N, C, H, W, K, ks = 2, 16, 11, 11, 72, 3
+    rng = np.random.default_rng(77)
+    w = sparse_filter(rng, K, C, ks, 0.8)
+    x = relu_like(rng, (N, C, H, W))
+    sf = T.SparseFilter(w, C, K, ks, 32, True, True, T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL)
+    order = sf.oc_permutation_
+    assert sorted(order.tolist()) == list(range(K)) and order.tolist() != list(range(K))
+    pk = T.G950Filter(w, 8, oc_order=order)
+    a, o = pk.host_arrays(), O.G950Pack(w, 8, order)
+    assert np.array_equal(a["position"], o.position) and np.array_equal(a["oc_order"], o.order)
+    y = run_conv(T, torch, pk, x, K, ks, 1, 1)
+    assert max_rel_err(y, O.host_conv2d(x, w, 1, 1, threads=4)) <= TOL
+    with pytest.raises(T.TetrisError):
+        T.G950Filter(w, 8, oc_order=np.zeros(K, np.int32))
+
+
+def test_reference_shaped_entry_points(env):
+    T, torch, O = env
+    N, C, H, W, K, ks, stride, pad = 2, 24, 20, 20, 48, 3, 1, 1
+    rng = np.random.default_rng(11)
+    w = sparse_filter(rng, K, C, ks, 0.85)
+    x = relu_like(rng, (N, C, H, W))
+    ref = O.host_conv2d(x, w, stride, pad, threads=4)
+    for fn in (T.CudaSparseConv2d, T.SparseConv2d_SPF):
+        for reorder in (True, False):
+            y, ms = fn(x, w, N, H, W, C, K, ks, stride, pad, 0, "NHWC", reorder)
+            assert ms > 0 and max_rel_err(y, ref) <= TOL
+    # raw launcher with a SparseFilter's device arrays, as the reference's mains call it
+    sf = T.SparseFilter(w, C, K, ks, 128, True, True, T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL)
+    dx = torch.from_numpy(x).cuda()
+    dy = torch.zeros((N, K, H, W), device="cuda")
+    T.SparseConv2d(dx.data_ptr(), sf.GetDeviceOffsets(), sf.GetDeviceStageLen(), sf.GetDeviceOCPermutation(),
+                   sf.GetDevicePosition(), sf.GetDeviceValues(), dy.data_ptr(), N, H, W, C, K, ks, stride, pad)
+    torch.cuda.synchronize()
+    assert max_rel_err(dy.cpu().numpy(), ref) <= TOL
+    # the device copies hold the same bytes as the host vectors
+    dev_vals = torch.empty(len(sf.values_), device="cuda")
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipMemcpy(ctypes.c_void_p(dev_vals.data_ptr()), ctypes.c_void_p(sf.GetDeviceValues()),
+                  ctypes.c_size_t(4 * len(sf.values_)), 3)
+    assert dev_vals.cpu().numpy().tobytes() == sf.values_.tobytes()
+    with pytest.raises(T.TetrisError) as e:
+        T.SparseConv2d(dx.data_ptr(), 0, 0, 0, 0, dx.data_ptr(), dy.data_ptr(), N, H, W, C, K, ks, stride, pad)
+    assert e.value.code == T.ENOTFOUND
+
+
+@pytest.mark.parametrize("name", ["rn90_3x3", "rn90_stem", "rn98_1x1", "vgg_64x128", "yolo_255"])
+def test_shipped_pruned_layers(env, name):
+    # real magnitude-pruned weights: very uneven rows, channels with no weights at all, K = 255
+    T, torch, O = env
+    hdr, w, _ = golden_weights(name)
+    N = 2
+    H = min(hdr["H"], 40)
+    rng = np.random.default_rng(5)
+    x = relu_like(rng, (N, hdr["IC"], H, H))
+    y, _ = T.CudaSparseConv2d(x, w, N, H, H, hdr["IC"], hdr["OC"], hdr["KS"], hdr["STRIDE"], hdr["PAD"])
+    ref = O.host_conv2d(x, w, hdr["STRIDE"], hdr["PAD"], threads=8)
+    assert max_rel_err(y, ref) <= TOL
+
+
+def test_config1_full_size(env):
+    # BASELINE config 1: N=1, C=64, 56x56, K=128, 3x3/s1/p1, 90 % sparse
+    T, torch, O = env
+    from tetris_amd import workloads as W
+
+    L = W.single_layer()[0]
+    w, x = W.make_weights(L), W.make_activations(L, 1)
+    assert int((w != 0).sum()) == 7373
+    tile = T.tile_select(1, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+    pk = T.G950Filter(w, tile.tile_ic)
+    y = run_conv(T, torch, pk, x, L.K, L.ks, L.stride, L.pad, tile)
+    ref = O.host_conv2d(x, w, L.stride, L.pad, threads=8)
+    assert max_rel_err(y, ref) <= TOL
+    if O.ref_available():
+        assert max_rel_err(y, O.ref_host_conv2d(x, w, L.stride, L.pad)) <= TOL
+
+
+def test_full_size_properties(env):
+    # At sizes the CPU cannot check densely: linearity in the filter, and a slice checked against the oracle.
+    T, torch, O = env
+    from tetris_amd import workloads as W
+
+    L = W.vgg19()[5]  # 256 -> 256 at 56x56
+    N = 16
+    w, x = W.make_weights(L), W.make_activations(L, N)
+    tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+    rng = np.random.default_rng(1)
+    mask = rng.random(w.shape) < 0.5
+    wa, wb = np.where(mask, w, 0).astype(np.float32), np.where(mask, 0, w).astype(np.float32)
+    ys = []
+    dx = torch.from_numpy(x).cuda()
+    for part in (w, wa, wb):
+        pk = T.G950Filter(part, tile.tile_ic)
+        dy = torch.empty((N, L.K, 56, 56), device="cuda")
+        pk.launch(dx.data_ptr(), dy.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
+        torch.cuda.synchronize()
+        ys.append(dy)
+    err = (ys[0] - (ys[1] + ys[2])).abs() / ys[0].abs().clamp_min(max(1e-3, 1e-2 * float(ys[0].abs().max())))
+    assert float(err.max()) <= TOL
+    # one image, a few output channels, against the dense oracle
+    sel = [0, 1, 127, 255]
+    ref = O.host_conv2d(x[3:4], w[sel], L.stride, L.pad, threads=8)
+    assert max_rel_err(ys[0][3:4, sel].cpu().numpy(), ref) <= TOL

@@ -1,0 +1,339 @@
+// extern "C" layer of libtetris_spconv2d.so: handles, launch, the reference-shaped host entry points
+// (CudaSparseConv2d, Tetris/spconv2d.cc:332-367; SparseConv2d_SPF, Tetris/spf.cc:22-93) and the path's
+// small utilities (Tetris/tensor_utils.cc:17-34, :55-82).
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+
+#include "common.h"
+
+namespace tetris {
+
+namespace {
+thread_local std::string g_error;
+
+std::mutex g_registry_mu;
+std::map<const void*, tetris_spf*> g_registry;  // d_values of every live tetris_spf -> its handle
+}  // namespace
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_error = buf;
+  return code;
+}
+
+namespace {
+
+template <typename T>
+int upload(const std::vector<T>& v, T** d) {
+  *d = nullptr;
+  const size_t bytes = std::max<size_t>(v.size(), 1) * sizeof(T);
+  TETRIS_HIP(hipMalloc(d, bytes));
+  if (!v.empty()) TETRIS_HIP(hipMemcpy(*d, v.data(), v.size() * sizeof(T), hipMemcpyHostToDevice));
+  return TETRIS_OK;
+}
+
+int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
+               const tetris_tile* tile, hipStream_t stream) {
+  if (!p || !d_in || !d_out) return fail(TETRIS_EINVAL, "null argument");
+  tetris_tile t{};
+  if (tile && tile->lanes_w > 0) {
+    t = *tile;
+  } else {
+    int rc = choose_tile(N, H, W, p->C, p->K, p->ks, stride, pad, &t);
+    if (rc) return rc;
+  }
+  Geom g;
+  int rc = make_geom(p, N, H, W, stride, pad, t, &g);
+  if (rc) return rc;
+  const int2* entries = nullptr;
+  rc = g950_bind(p, g, stream, &entries);
+  if (rc) return rc;
+  return launch_conv(g, t, d_in, d_out, entries, p->d_seg_off, p->d_oc_order, stream);
+}
+
+int time_launches(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
+                  const tetris_tile* tile, hipStream_t stream, int warm, int repeat, float* ms_out) {
+  if (repeat <= 0 || warm < 0) return fail(TETRIS_EINVAL, "bad warm/repeat");
+  hipEvent_t a, b;
+  TETRIS_HIP(hipEventCreate(&a));
+  TETRIS_HIP(hipEventCreate(&b));
+  int rc = TETRIS_OK;
+  for (int i = 0; i < warm && rc == TETRIS_OK; ++i) rc = run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, stream);
+  if (rc == TETRIS_OK) {
+    TETRIS_HIP(hipStreamSynchronize(stream));
+    TETRIS_HIP(hipEventRecord(a, stream));
+    for (int i = 0; i < repeat && rc == TETRIS_OK; ++i)
+      rc = run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, stream);
+    TETRIS_HIP(hipEventRecord(b, stream));
+    TETRIS_HIP(hipEventSynchronize(b));
+    float ms = 0;
+    TETRIS_HIP(hipEventElapsedTime(&ms, a, b));
+    if (ms_out) *ms_out = ms / repeat;
+  }
+  (void)hipEventDestroy(a);
+  (void)hipEventDestroy(b);
+  return rc;
+}
+
+// Shared body of the two host-to-host entry points.
+int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K, int ks,
+              int stride, int pad, hipStream_t stream, bool apply_reorder, bool fixed_spf_config, float* ms_out) {
+  if (!h_in || !h_filter || !h_out) return fail(TETRIS_EINVAL, "null argument");
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
+    return fail(TETRIS_EINVAL, "bad conv shape");
+  const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
+  if (OH <= 0 || OW <= 0) return fail(TETRIS_EINVAL, "empty output");
+  tetris_tile tile{};
+  int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &tile);
+  if (rc) return rc;
+  // The spf entry point of the reference fixes TILE_IC = 128 and never regroups differently per tile;
+  // here it fixes the packer arguments the same way and leaves the kernel tile to the selector.
+  const int ref_tile_ic = fixed_spf_config ? 128 : 32;
+  tetris_spf* spf = nullptr;
+  std::vector<int32_t> order;
+  if (apply_reorder) {
+    // keep the reference's output-channel regrouping for the slot order of the kernel's pack
+    rc = tetris_spf_create(h_filter, C, K, ks, ref_tile_ic, 1, 1, TETRIS_REORDER_OUT_CHANNEL, &spf);
+    if (rc) return rc;
+    order = spf->oc_permutation;
+  }
+  tetris_g950* pack = nullptr;
+  rc = tetris_g950_create(h_filter, C, K, ks, tile.tile_ic, apply_reorder ? order.data() : nullptr, stream, &pack);
+  float *d_in = nullptr, *d_out = nullptr;
+  const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
+  auto done = [&](int code) {
+    if (d_in) (void)hipFree(d_in);
+    if (d_out) (void)hipFree(d_out);
+    tetris_g950_destroy(pack);
+    tetris_spf_destroy(spf);
+    return code;
+  };
+  if (rc) return done(rc);
+#define HIPD(call)                                                                                          \
+  do {                                                                                                      \
+    hipError_t e_ = (call);                                                                                 \
+    if (e_ != hipSuccess)                                                                                   \
+      return done(fail(TETRIS_EHIP, "%s failed at %s:%d: %s", #call, __FILE__, __LINE__, hipGetErrorString(e_))); \
+  } while (0)
+  HIPD(hipMalloc(&d_in, in_bytes));
+  HIPD(hipMalloc(&d_out, out_bytes));
+  HIPD(hipMemcpyAsync(d_in, h_in, in_bytes, hipMemcpyHostToDevice, stream));
+  float ms = 0;
+  rc = time_launches(pack, d_in, d_out, N, H, W, stride, pad, &tile, stream, 30, 100, &ms);
+  if (rc) return done(rc);
+  HIPD(hipMemcpyAsync(h_out, d_out, out_bytes, hipMemcpyDeviceToHost, stream));
+  HIPD(hipStreamSynchronize(stream));
+#undef HIPD
+  if (ms_out) *ms_out = ms;
+  return done(TETRIS_OK);
+}
+
+}  // namespace
+}  // namespace tetris
+
+using namespace tetris;
+
+extern "C" {
+
+const char* tetris_last_error(void) { return g_error.c_str(); }
+const char* tetris_version(void) { return "tetris-spconv2d gfx950 0.1"; }
+
+// Device copies of the five arrays are made on first use, so that packing alone needs no GPU.
+static int spf_ensure_device(tetris_spf* f) {
+  std::lock_guard<std::mutex> lock(f->mu);
+  if (f->d_values) return TETRIS_OK;
+  int rc = upload(f->offsets, &f->d_offsets);
+  if (rc == TETRIS_OK) rc = upload(f->stage_len, &f->d_stage_len);
+  if (rc == TETRIS_OK) rc = upload(f->position, &f->d_position);
+  if (rc == TETRIS_OK) rc = upload(f->oc_permutation, &f->d_oc_permutation);
+  float* d_values = nullptr;
+  if (rc == TETRIS_OK) rc = upload(f->values, &d_values);
+  if (rc != TETRIS_OK) {
+    if (f->d_offsets) (void)hipFree(f->d_offsets);
+    if (f->d_stage_len) (void)hipFree(f->d_stage_len);
+    if (f->d_position) (void)hipFree(f->d_position);
+    if (f->d_oc_permutation) (void)hipFree(f->d_oc_permutation);
+    f->d_offsets = f->d_stage_len = f->d_position = f->d_oc_permutation = nullptr;
+    return rc;
+  }
+  f->d_values = d_values;
+  std::lock_guard<std::mutex> rlock(g_registry_mu);
+  g_registry[f->d_values] = f;
+  return TETRIS_OK;
+}
+
+// The kernel's own pack of this filter for `tile_ic` staged input channels, in the same slot order.
+static int spf_kernel_pack(tetris_spf* f, int tile_ic, hipStream_t stream, tetris_g950** out) {
+  std::lock_guard<std::mutex> lock(f->mu);
+  auto it = f->kernel_packs.find(tile_ic);
+  if (it == f->kernel_packs.end()) {
+    tetris_g950* p = nullptr;
+    int rc = tetris_g950_create(f->filter.data(), f->C, f->K, f->ks, tile_ic, f->oc_permutation.data(), stream, &p);
+    if (rc) return rc;
+    it = f->kernel_packs.emplace(tile_ic, p).first;
+  }
+  *out = it->second;
+  return TETRIS_OK;
+}
+
+int tetris_spf_create(const float* h_filter, int C, int K, int ks, int tile_ic, int apply_reorder, int apply_vectorize,
+                      unsigned flags, tetris_spf** out) {
+  if (!out) return fail(TETRIS_EINVAL, "null argument");
+  tetris_spf* f = new tetris_spf;
+  int rc = spf_pack_host(h_filter, C, K, ks, tile_ic, apply_reorder != 0, apply_vectorize != 0, flags, f);
+  if (rc != TETRIS_OK) {
+    delete f;
+    return rc;
+  }
+  f->filter.assign(h_filter, h_filter + (size_t)C * K * ks * ks);  // the kernel's packs are made from it at launch
+  *out = f;
+  return TETRIS_OK;
+}
+
+void tetris_spf_destroy(tetris_spf* f) {
+  if (!f) return;
+  if (f->d_values) {
+    std::lock_guard<std::mutex> lock(g_registry_mu);
+    auto it = g_registry.find(f->d_values);
+    if (it != g_registry.end() && it->second == f) g_registry.erase(it);
+  }
+  for (auto& kv : f->kernel_packs) tetris_g950_destroy(kv.second);
+  if (f->d_offsets) (void)hipFree(f->d_offsets);
+  if (f->d_stage_len) (void)hipFree(f->d_stage_len);
+  if (f->d_position) (void)hipFree(f->d_position);
+  if (f->d_values) (void)hipFree(f->d_values);
+  if (f->d_oc_permutation) (void)hipFree(f->d_oc_permutation);
+  delete f;
+}
+
+int tetris_spf_host_arrays(const tetris_spf* f, tetris_spf_arrays* o) {
+  if (!f || !o) return fail(TETRIS_EINVAL, "null argument");
+  o->offsets = f->offsets.data();               o->n_offsets = (int64_t)f->offsets.size();
+  o->stage_len = f->stage_len.data();           o->n_stage_len = (int64_t)f->stage_len.size();
+  o->position = f->position.data();             o->n_position = (int64_t)f->position.size();
+  o->values = f->values.data();                 o->n_values = (int64_t)f->values.size();
+  o->oc_permutation = f->oc_permutation.data(); o->n_oc_permutation = (int64_t)f->oc_permutation.size();
+  o->nnz = f->nnz;
+  o->tile_ic = f->tile_ic;
+  return TETRIS_OK;
+}
+
+int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* o) {
+  int rc = tetris_spf_host_arrays(f, o);
+  if (rc) return rc;
+  rc = spf_ensure_device(f);
+  if (rc) return rc;
+  o->offsets = f->d_offsets;
+  o->stage_len = f->d_stage_len;
+  o->position = f->d_position;
+  o->values = f->d_values;
+  o->oc_permutation = f->d_oc_permutation;
+  return TETRIS_OK;
+}
+
+int tetris_tile_select(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* out) {
+  if (!out) return fail(TETRIS_EINVAL, "null argument");
+  return choose_tile(N, H, W, C, K, ks, stride, pad, out);
+}
+
+int tetris_spconv2d_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
+                           const tetris_tile* tile, void* stream) {
+  return run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, static_cast<hipStream_t>(stream));
+}
+
+int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,
+                               const int32_t* d_perm, const int32_t* d_position, const float* d_values, float* d_out,
+                               int N, int H, int W, int C, int K, int ks, int stride, int pad, void* stream) {
+  (void)d_offsets; (void)d_stage_len; (void)d_perm; (void)d_position;
+  tetris_spf* f = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_registry_mu);
+    auto it = g_registry.find(d_values);
+    if (it != g_registry.end()) f = it->second;
+  }
+  if (!f) return fail(TETRIS_ENOTFOUND, "device arrays do not belong to a live tetris_spf handle");
+  if (f->C != C || f->K != K || f->ks != ks)
+    return fail(TETRIS_EINVAL, "shape C=%d K=%d ks=%d does not match the packed filter (%d, %d, %d)", C, K, ks, f->C,
+                f->K, f->ks);
+  tetris_tile t{};
+  int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &t);
+  if (rc) return rc;
+  tetris_g950* pack = nullptr;
+  rc = spf_kernel_pack(f, t.tile_ic, static_cast<hipStream_t>(stream), &pack);
+  if (rc) return rc;
+  return run_launch(pack, d_in, d_out, N, H, W, stride, pad, &t, static_cast<hipStream_t>(stream));
+}
+
+int tetris_spconv2d_time(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
+                         const tetris_tile* tile, void* stream, int warm, int repeat, float* ms_out) {
+  return time_launches(p, d_in, d_out, N, H, W, stride, pad, tile, static_cast<hipStream_t>(stream), warm, repeat,
+                       ms_out);
+}
+
+int tetris_spconv2d_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K,
+                         int ks, int stride, int pad, void* stream, const char* layout, int apply_reorder,
+                         float* ms_out) {
+  (void)layout;
+  return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream),
+                   apply_reorder != 0, false, ms_out);
+}
+
+int tetris_spconv2d_spf_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K,
+                             int ks, int stride, int pad, void* stream, const char* layout, int apply_reorder,
+                             float* ms_out) {
+  (void)layout;
+  return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream),
+                   apply_reorder != 0, true, ms_out);
+}
+
+int tetris_read_weight_file(const char* path, int32_t header[8], float** h_filter_out, int64_t* nnz_out) {
+  if (!path || !header || !h_filter_out) return fail(TETRIS_EINVAL, "null argument");
+  FILE* fp = fopen(path, "r");
+  if (!fp) return fail(TETRIS_EIO, "Open file error: %s", path);
+  for (int i = 0; i < 8; ++i)
+    if (fscanf(fp, "%d", &header[i]) != 1) {
+      fclose(fp);
+      return fail(TETRIS_EIO, "truncated header in %s", path);
+    }
+  const int64_t n = (int64_t)header[3] * header[2] * header[4] * header[4];
+  if (n <= 0 || header[4] > kMaxKs) {
+    fclose(fp);
+    return fail(TETRIS_EINVAL, "bad header in %s", path);
+  }
+  float* f = static_cast<float*>(malloc(sizeof(float) * (size_t)n));
+  if (!f) {
+    fclose(fp);
+    return fail(TETRIS_EINVAL, "out of memory for %lld weights", (long long)n);
+  }
+  int64_t nnz = 0;
+  for (int64_t i = 0; i < n; ++i) {
+    if (fscanf(fp, "%f", &f[i]) != 1) {
+      free(f);
+      fclose(fp);
+      return fail(TETRIS_EIO, "truncated weights in %s (%lld of %lld)", path, (long long)i, (long long)n);
+    }
+    nnz += f[i] != 0;
+  }
+  fclose(fp);
+  *h_filter_out = f;
+  if (nnz_out) *nnz_out = nnz;
+  return TETRIS_OK;
+}
+
+void tetris_free(void* p) { free(p); }
+
+int tetris_float_equal(float x, float y) { return std::fabs(x - y) <= 1e-5 * (std::fabs(x) + std::fabs(y)) + 1e-5; }
+
+int64_t tetris_tensor_first_mismatch(const float* x, const float* y, int64_t len) {
+  for (int64_t i = 0; i < len; ++i)
+    if (!tetris_float_equal(x[i], y[i])) return i;
+  return -1;
+}
+
+}  // extern "C"

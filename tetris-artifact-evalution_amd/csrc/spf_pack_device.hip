@@ -1,0 +1,267 @@
+// gfx950 weight-preprocessing pass: dense OIHW fp32 filter -> per-(slot, stage) runs of non-zero
+// (position, value) entries, built on the device in three deterministic kernels (count, scan, scatter).
+//
+// Takes the place of the reference's host-side SparseFilter constructor (Tetris/spconv2d_utils.h:62-98,
+// :206-244) for the HIP kernel.  The position word keeps the reference encoding
+// s | r << 3 | (ic % tile_ic) << 6 (spconv2d_utils.h:91) and the zero test keeps `value != 0.f`, so -0.0
+// is dropped like the reference drops it.  What differs is the arrangement: the reference interleaves 32
+// lanes x 4 entries because its lanes are output channels; here every entry is wave-uniform, so a run
+// belongs to one output channel and is padded to a multiple of 8 entries (one 64-byte scalar fetch).
+#include "common.h"
+
+namespace tetris {
+namespace {
+
+// one wave per (slot, stage): the stage's weights are cs*ks*ks consecutive floats
+__global__ __launch_bounds__(256) void count_kernel(const float* __restrict__ filter, const int32_t* __restrict__ oc_order,
+                                                    int32_t* __restrict__ seg_nnz, int32_t* __restrict__ seg_pad, int C,
+                                                    int ks, int tile_ic, int stages, int nseg) {
+  const int seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (seg >= nseg) return;
+  const int slot = seg / stages, st = seg - slot * stages;
+  const int oc = oc_order[slot];
+  int cnt = 0;
+  if (oc >= 0) {
+    const int kk = ks * ks;
+    const int c0 = st * tile_ic;
+    const int n = min(tile_ic, C - c0) * kk;
+    const float* src = filter + ((size_t)oc * C + c0) * kk;
+    for (int i = lane; i < n; i += 64) cnt += (src[i] != 0.f) ? 1 : 0;
+    for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+  }
+  if (lane == 0) {
+    seg_nnz[seg] = cnt;
+    seg_pad[seg] = (cnt + kBatch - 1) / kBatch * kBatch;
+  }
+}
+
+// exclusive scan of seg_pad into seg_off[0..n], single workgroup
+__global__ __launch_bounds__(1024) void scan_kernel(const int32_t* __restrict__ seg_pad, int32_t* __restrict__ seg_off,
+                                                    int n) {
+  __shared__ int part[1024];
+  const int tid = threadIdx.x;
+  const int chunk = (n + 1023) / 1024;
+  const int b = tid * chunk, e = min(n, b + chunk);
+  int s = 0;
+  for (int i = b; i < e; ++i) s += seg_pad[i];
+  part[tid] = s;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {
+    const int v = tid >= off ? part[tid - off] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = tid ? part[tid - 1] : 0;
+  for (int i = b; i < e; ++i) {
+    seg_off[i] = run;
+    run += seg_pad[i];
+  }
+  if (tid == 1023) seg_off[n] = part[1023];
+}
+
+__global__ __launch_bounds__(256) void scatter_kernel(const float* __restrict__ filter,
+                                                      const int32_t* __restrict__ oc_order,
+                                                      const int32_t* __restrict__ seg_off, int32_t* __restrict__ position,
+                                                      float* __restrict__ values, int C, int ks, int tile_ic, int stages,
+                                                      int nseg) {
+  const int seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (seg >= nseg) return;
+  const int slot = seg / stages, st = seg - slot * stages;
+  const int oc = oc_order[slot];
+  const int beg = seg_off[seg], end = seg_off[seg + 1];
+  int written = 0;
+  if (oc >= 0) {
+    const int kk = ks * ks;
+    const int c0 = st * tile_ic;
+    const int n = min(tile_ic, C - c0) * kk;
+    const float* src = filter + ((size_t)oc * C + c0) * kk;
+    for (int i0 = 0; i0 < n; i0 += 64) {
+      const int i = i0 + lane;
+      const float v = i < n ? src[i] : 0.f;
+      const bool nz = v != 0.f;
+      const unsigned long long m = __ballot(nz);
+      if (nz) {
+        const int rank = __popcll(m & ((1ull << lane) - 1ull));
+        const int ic = i / kk, rs = i - ic * kk;
+        const int r = rs / ks, s = rs - r * ks;
+        position[beg + written + rank] = s + (r << 3) + (ic << 6);
+        values[beg + written + rank] = v;
+      }
+      written += __popcll(m);
+    }
+  }
+  for (int i = beg + written + lane; i < end; i += 64) {  // padding entries
+    position[i] = 0;
+    values[i] = 0.f;
+  }
+}
+
+__global__ __launch_bounds__(256) void bind_kernel(const int32_t* __restrict__ position, const float* __restrict__ values,
+                                                   int2* __restrict__ out, long long n, int plane, int pitch, int par,
+                                                   int stride) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int pos = position[i];
+  const int s = pos & 7, r = (pos >> 3) & 7, ic = pos >> 6;
+  int2 e;
+  e.x = 4 * (ic * plane + r * pitch + (s % stride) * par + (s / stride) * 4);
+  e.y = __float_as_int(values[i]);
+  out[i] = e;
+}
+
+int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, const int32_t* oc_order, hipStream_t stream,
+                tetris_g950** out) {
+  if (!d_filter || !out) return fail(TETRIS_EINVAL, "null argument");
+  if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || tile_ic <= 0)
+    return fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d tile_ic=%d (ks <= %d)", C, K, ks, tile_ic, kMaxKs);
+  tetris_g950* p = new tetris_g950;
+  p->C = C; p->K = K; p->ks = ks; p->tile_ic = tile_ic;
+  p->stages = (C - 1) / tile_ic + 1;
+  p->slots = (K + 127) / 128 * 128;
+  const int nseg = p->slots * p->stages;
+
+  std::vector<int32_t> order(p->slots, -1);
+  std::vector<char> seen(K, 0);
+  for (int i = 0; i < K; ++i) {
+    const int oc = oc_order ? oc_order[i] : i;
+    if (oc < 0 || oc >= K || seen[oc]) {
+      delete p;
+      return fail(TETRIS_EINVAL, "oc_order is not a permutation of 0..%d", K - 1);
+    }
+    seen[oc] = 1;
+    order[i] = oc;
+  }
+  int32_t* d_pad = nullptr;
+  auto cleanup = [&](int rc) {
+    if (d_pad) (void)hipFree(d_pad);
+    if (rc != TETRIS_OK) tetris_g950_destroy(p);
+    return rc;
+  };
+#define HIPC(call)                                                                                              \
+  do {                                                                                                          \
+    hipError_t e_ = (call);                                                                                     \
+    if (e_ != hipSuccess)                                                                                       \
+      return cleanup(fail(TETRIS_EHIP, "%s failed at %s:%d: %s", #call, __FILE__, __LINE__, hipGetErrorString(e_))); \
+  } while (0)
+  HIPC(hipMalloc(&p->d_oc_order, sizeof(int32_t) * p->slots));
+  HIPC(hipMalloc(&p->d_seg_off, sizeof(int32_t) * (nseg + 1)));
+  HIPC(hipMalloc(&p->d_seg_nnz, sizeof(int32_t) * nseg));
+  HIPC(hipMalloc(&d_pad, sizeof(int32_t) * nseg));
+  HIPC(hipMemcpyAsync(p->d_oc_order, order.data(), sizeof(int32_t) * p->slots, hipMemcpyHostToDevice, stream));
+  const int blocks = (nseg + 3) / 4;
+  hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, stream, d_filter, p->d_oc_order, p->d_seg_nnz, d_pad, C,
+                     ks, tile_ic, p->stages, nseg);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, d_pad, p->d_seg_off, nseg);
+  HIPC(hipGetLastError());
+  int32_t total = 0;
+  HIPC(hipMemcpyAsync(&total, p->d_seg_off + nseg, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+  HIPC(hipStreamSynchronize(stream));
+  p->n_entries = total;
+  // one spare batch so that a kernel may prefetch the batch after the last one
+  HIPC(hipMalloc(&p->d_position, sizeof(int32_t) * (size_t)(total + kBatch)));
+  HIPC(hipMalloc(&p->d_values, sizeof(float) * (size_t)(total + kBatch)));
+  HIPC(hipMemsetAsync(p->d_position + total, 0, sizeof(int32_t) * kBatch, stream));
+  HIPC(hipMemsetAsync(p->d_values + total, 0, sizeof(float) * kBatch, stream));
+  hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(256), 0, stream, d_filter, p->d_oc_order, p->d_seg_off,
+                     p->d_position, p->d_values, C, ks, tile_ic, p->stages, nseg);
+  HIPC(hipGetLastError());
+  // nnz = sum of seg_nnz, summed on the host (small)
+  std::vector<int32_t> nz(nseg);
+  HIPC(hipMemcpyAsync(nz.data(), p->d_seg_nnz, sizeof(int32_t) * nseg, hipMemcpyDeviceToHost, stream));
+  HIPC(hipStreamSynchronize(stream));
+  p->nnz = 0;
+  for (int v : nz) p->nnz += v;
+#undef HIPC
+  *out = p;
+  return cleanup(TETRIS_OK);
+}
+
+}  // namespace
+
+int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** entries_out) {
+  const BoundKey key{g.plane, g.pitch, g.par, g.stride};
+  std::lock_guard<std::mutex> lock(p->mu);
+  auto it = p->bound.find(key);
+  if (it == p->bound.end()) {
+    int2* d = nullptr;
+    const long long n = p->n_entries + kBatch;
+    TETRIS_HIP(hipMalloc(&d, sizeof(int2) * (size_t)n));
+    hipLaunchKernelGGL(bind_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p->d_position, p->d_values,
+                       d, n, g.plane, g.pitch, g.par, g.stride);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      (void)hipFree(d);
+      return fail(TETRIS_EHIP, "bind_kernel launch failed: %s", hipGetErrorString(e));
+    }
+    it = p->bound.emplace(key, d).first;
+  }
+  *entries_out = it->second;
+  return TETRIS_OK;
+}
+
+}  // namespace tetris
+
+extern "C" {
+
+int tetris_g950_create_device(const float* d_filter, int C, int K, int ks, int tile_ic, const int32_t* oc_order,
+                              void* stream, tetris_g950** out) {
+  return tetris::pack_device(d_filter, C, K, ks, tile_ic, oc_order, static_cast<hipStream_t>(stream), out);
+}
+
+int tetris_g950_create(const float* h_filter, int C, int K, int ks, int tile_ic, const int32_t* oc_order, void* stream,
+                       tetris_g950** out) {
+  if (!h_filter) return tetris::fail(TETRIS_EINVAL, "null filter");
+  if (C <= 0 || K <= 0 || ks <= 0) return tetris::fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d", C, K, ks);
+  float* d = nullptr;
+  const size_t bytes = sizeof(float) * (size_t)C * K * ks * ks;
+  TETRIS_HIP(hipMalloc(&d, bytes));
+  hipError_t e = hipMemcpyAsync(d, h_filter, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream));
+  int rc = e == hipSuccess ? TETRIS_OK : tetris::fail(TETRIS_EHIP, "filter upload failed: %s", hipGetErrorString(e));
+  if (rc == TETRIS_OK) rc = tetris::pack_device(d, C, K, ks, tile_ic, oc_order, static_cast<hipStream_t>(stream), out);
+  (void)hipStreamSynchronize(static_cast<hipStream_t>(stream));
+  (void)hipFree(d);
+  return rc;
+}
+
+void tetris_g950_destroy(tetris_g950* p) {
+  if (!p) return;
+  for (auto& kv : p->bound) (void)hipFree(kv.second);
+  (void)hipFree(p->d_seg_off);
+  (void)hipFree(p->d_seg_nnz);
+  (void)hipFree(p->d_position);
+  (void)hipFree(p->d_values);
+  (void)hipFree(p->d_oc_order);
+  delete p;
+}
+
+int tetris_g950_host_arrays(tetris_g950* p, tetris_g950_arrays* out) {
+  if (!p || !out) return tetris::fail(TETRIS_EINVAL, "null argument");
+  const int nseg = p->slots * p->stages;
+  std::lock_guard<std::mutex> lock(p->mu);
+  if (p->h_seg_off.empty()) {
+    p->h_seg_off.resize(nseg + 1);
+    p->h_seg_nnz.resize(nseg);
+    p->h_position.resize(p->n_entries);
+    p->h_values.resize(p->n_entries);
+    p->h_oc_order.resize(p->slots);
+    TETRIS_HIP(hipMemcpy(p->h_seg_off.data(), p->d_seg_off, sizeof(int32_t) * (nseg + 1), hipMemcpyDeviceToHost));
+    TETRIS_HIP(hipMemcpy(p->h_seg_nnz.data(), p->d_seg_nnz, sizeof(int32_t) * nseg, hipMemcpyDeviceToHost));
+    if (p->n_entries) {
+      TETRIS_HIP(hipMemcpy(p->h_position.data(), p->d_position, sizeof(int32_t) * p->n_entries, hipMemcpyDeviceToHost));
+      TETRIS_HIP(hipMemcpy(p->h_values.data(), p->d_values, sizeof(float) * p->n_entries, hipMemcpyDeviceToHost));
+    }
+    TETRIS_HIP(hipMemcpy(p->h_oc_order.data(), p->d_oc_order, sizeof(int32_t) * p->slots, hipMemcpyDeviceToHost));
+  }
+  out->seg_offsets = p->h_seg_off.data(); out->n_seg_offsets = nseg + 1;
+  out->seg_nnz = p->h_seg_nnz.data();     out->n_seg_nnz = nseg;
+  out->position = p->h_position.data();   out->n_entries = p->n_entries;
+  out->values = p->h_values.data();
+  out->oc_order = p->h_oc_order.data();   out->n_slots = p->slots;
+  out->stages = p->stages; out->tile_ic = p->tile_ic; out->nnz = p->nnz;
+  return TETRIS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,306 @@
+"""Python face of libtetris_spconv2d.so (ctypes over the C ABI in include/tetris_spconv2d.h).
+
+The names mirror the reference's C++ interface for this path so that tests read like its mains:
+SparseFilter (Tetris/spconv2d_utils.h:23-515), SparseConv2d (Tetris/spconv2d_kernel.cuh:14-21),
+CudaSparseConv2d (Tetris/spconv2d.cc:332-367), SparseConv2d_SPF (Tetris/spf.cc:22-93).
+PyTorch, where used by callers, only provides device memory and streams; nothing here imports it.
+There is no CPU fallback: if the library is missing, importing this module fails.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libtetris_spconv2d.so")
+if not os.path.exists(LIB_PATH):
+    raise ImportError("libtetris_spconv2d.so is not built: run `make -C tetris-artifact-evalution_amd` "
+                      "(or __graft_entry__.build())")
+
+
+def _share_hip_runtime_with_torch():
+    """A process can hold one HIP runtime.  PyTorch-ROCm wheels bundle their own libamdhip64 (same soname as
+    the system one); if this library were loaded first it would bind the system copy and a later
+    `import torch` would bring in a second runtime that finds no device.  So when torch is installed and not
+    yet loaded, its copy is loaded first and both sides resolve to it."""
+    import importlib.util
+    import sys
+
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.submodule_search_locations:
+        return
+    bundled = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+    if os.path.exists(bundled):
+        C.CDLL(bundled, mode=C.RTLD_GLOBAL)
+
+
+_share_hip_runtime_with_torch()
+_lib = C.CDLL(LIB_PATH)
+
+BANK_OPTIMIZE = 1
+REORDER_OUT_CHANNEL = 2
+
+OK, EINVAL, EHIP, EUNSUPPORTED, ENOTFOUND, EIO = range(6)
+
+
+class TetrisError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("tetris error %d: %s" % (code, msg))
+        self.code = code
+
+
+class _SpfArrays(C.Structure):
+    _fields_ = [("offsets", C.c_void_p), ("n_offsets", C.c_int64), ("stage_len", C.c_void_p), ("n_stage_len", C.c_int64),
+                ("position", C.c_void_p), ("n_position", C.c_int64), ("values", C.c_void_p), ("n_values", C.c_int64),
+                ("oc_permutation", C.c_void_p), ("n_oc_permutation", C.c_int64), ("nnz", C.c_int64),
+                ("tile_ic", C.c_int32)]
+
+
+class _G950Arrays(C.Structure):
+    _fields_ = [("seg_offsets", C.c_void_p), ("n_seg_offsets", C.c_int64), ("seg_nnz", C.c_void_p),
+                ("n_seg_nnz", C.c_int64), ("position", C.c_void_p), ("n_entries", C.c_int64), ("values", C.c_void_p),
+                ("oc_order", C.c_void_p), ("n_slots", C.c_int64), ("stages", C.c_int32), ("tile_ic", C.c_int32),
+                ("nnz", C.c_int64)]
+
+
+class Tile(C.Structure):
+    """tetris_tile: lanes_w, quads, oc_per_wave, waves, tile_ic (all zero = let the library choose)."""
+    _fields_ = [("lanes_w", C.c_int32), ("quads", C.c_int32), ("oc_per_wave", C.c_int32), ("waves", C.c_int32),
+                ("tile_ic", C.c_int32)]
+
+    def __repr__(self):
+        return "Tile(lanes_w=%d, quads=%d, oc_per_wave=%d, waves=%d, tile_ic=%d)" % (
+            self.lanes_w, self.quads, self.oc_per_wave, self.waves, self.tile_ic)
+
+
+_f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
+_i32p_opt = C.c_void_p
+
+_lib.tetris_last_error.restype = C.c_char_p
+_lib.tetris_version.restype = C.c_char_p
+_lib.tetris_spf_create.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_uint,
+                                   C.POINTER(C.c_void_p)]
+_lib.tetris_spf_destroy.argtypes = [C.c_void_p]
+_lib.tetris_spf_destroy.restype = None
+_lib.tetris_spf_host_arrays.argtypes = [C.c_void_p, C.POINTER(_SpfArrays)]
+_lib.tetris_spf_device_arrays.argtypes = [C.c_void_p, C.POINTER(_SpfArrays)]
+_lib.tetris_g950_create.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, _i32p_opt, C.c_void_p,
+                                    C.POINTER(C.c_void_p)]
+_lib.tetris_g950_create_device.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _i32p_opt, C.c_void_p,
+                                           C.POINTER(C.c_void_p)]
+_lib.tetris_g950_destroy.argtypes = [C.c_void_p]
+_lib.tetris_g950_destroy.restype = None
+_lib.tetris_g950_host_arrays.argtypes = [C.c_void_p, C.POINTER(_G950Arrays)]
+_lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
+_lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile),
+                                                                                                C.c_void_p]
+_lib.tetris_spconv2d_launch_spf.argtypes = [C.c_void_p] * 7 + [C.c_int] * 8 + [C.c_void_p]
+_lib.tetris_spconv2d_time.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
+    C.POINTER(Tile), C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float)]
+for _n in ("tetris_spconv2d_host", "tetris_spconv2d_spf_host"):
+    getattr(_lib, _n).argtypes = [_f32p, _f32p, _f32p] + [C.c_int] * 8 + [C.c_void_p, C.c_char_p, C.c_int,
+                                                                          C.POINTER(C.c_float)]
+_lib.tetris_read_weight_file.argtypes = [C.c_char_p, C.POINTER(C.c_int32), C.POINTER(C.POINTER(C.c_float)),
+                                         C.POINTER(C.c_int64)]
+_lib.tetris_free.argtypes = [C.c_void_p]
+_lib.tetris_free.restype = None
+_lib.tetris_float_equal.argtypes = [C.c_float, C.c_float]
+_lib.tetris_tensor_first_mismatch.argtypes = [_f32p, _f32p, C.c_int64]
+_lib.tetris_tensor_first_mismatch.restype = C.c_int64
+
+
+def _check(rc):
+    if rc != 0:
+        raise TetrisError(rc, _lib.tetris_last_error().decode())
+
+
+def version():
+    return _lib.tetris_version().decode()
+
+
+def out_extent(size, pad, ks, stride):
+    return (size + 2 * pad - ks) // stride + 1
+
+
+def _np_view(ptr, n, dtype):
+    if not ptr or n == 0:
+        return np.zeros(0, dtype)
+    ct = C.c_float if dtype == np.float32 else C.c_int32
+    return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(ct)), shape=(int(n),)).copy()
+
+
+class SparseFilter:
+    """SparseFilter<float,int,int>(filter, in_channel, out_channel, kernel_size, TILE_IC=32,
+    apply_reorder=False, apply_vectorize=True); `flags` carries the reference's build macros."""
+
+    def __init__(self, filter, in_channel, out_channel, kernel_size, TILE_IC=32, apply_reorder=False,
+                 apply_vectorize=True, flags=0):
+        w = np.ascontiguousarray(filter, np.float32).reshape(out_channel, in_channel, kernel_size, kernel_size)
+        self._h = C.c_void_p()
+        _check(_lib.tetris_spf_create(w, in_channel, out_channel, kernel_size, TILE_IC, int(apply_reorder),
+                                      int(apply_vectorize), flags, C.byref(self._h)))
+        a = _SpfArrays()
+        _check(_lib.tetris_spf_host_arrays(self._h, C.byref(a)))
+        self.in_channel_, self.out_channel_, self.kernel_size_ = in_channel, out_channel, kernel_size
+        self.TILE_IC_ = int(a.tile_ic)
+        self.nnz_ = int(a.nnz)
+        self.offsets_ = _np_view(a.offsets, a.n_offsets, np.int32)
+        self.stage_len_ = _np_view(a.stage_len, a.n_stage_len, np.int32)
+        self.position_ = _np_view(a.position, a.n_position, np.int32)
+        self.values_ = _np_view(a.values, a.n_values, np.float32)
+        self.oc_permutation_ = _np_view(a.oc_permutation, a.n_oc_permutation, np.int32)
+        self._dev = None
+
+    def _device(self):
+        if self._dev is None:
+            a = _SpfArrays()
+            _check(_lib.tetris_spf_device_arrays(self._h, C.byref(a)))
+            self._dev = a
+        return self._dev
+
+    def GetDeviceOffsets(self):
+        return self._device().offsets
+
+    def GetDeviceStageLen(self):
+        return self._device().stage_len
+
+    def GetDeviceValues(self):
+        return self._device().values
+
+    def GetDevicePosition(self):
+        return self._device().position
+
+    def GetDeviceOCPermutation(self):
+        return self._device().oc_permutation
+
+    def GetTileIC(self):
+        return self.TILE_IC_
+
+    def arrays(self):
+        return (self.offsets_, self.stage_len_, self.position_, self.values_, self.oc_permutation_)
+
+    def close(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.tetris_spf_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+
+class G950Filter:
+    """The gfx950 pack the HIP kernel consumes (tetris_g950_create / _create_device)."""
+
+    def __init__(self, filter, tile_ic, oc_order=None, stream=0, device_ptr=None, shape=None):
+        if device_ptr is None:
+            w = np.ascontiguousarray(filter, np.float32)
+            K, Cc, ks, _ = w.shape
+        else:
+            K, Cc, ks, _ = shape
+        order = None if oc_order is None else np.ascontiguousarray(oc_order, np.int32)
+        optr = None if order is None else order.ctypes.data_as(C.c_void_p)
+        self._h = C.c_void_p()
+        if device_ptr is None:
+            _check(_lib.tetris_g950_create(w, Cc, K, ks, tile_ic, optr, C.c_void_p(stream), C.byref(self._h)))
+        else:
+            _check(_lib.tetris_g950_create_device(C.c_void_p(device_ptr), Cc, K, ks, tile_ic, optr, C.c_void_p(stream),
+                                                  C.byref(self._h)))
+        self.K, self.C, self.ks, self.tile_ic = K, Cc, ks, tile_ic
+
+    def host_arrays(self):
+        a = _G950Arrays()
+        _check(_lib.tetris_g950_host_arrays(self._h, C.byref(a)))
+        return dict(seg_offsets=_np_view(a.seg_offsets, a.n_seg_offsets, np.int32),
+                    seg_nnz=_np_view(a.seg_nnz, a.n_seg_nnz, np.int32),
+                    position=_np_view(a.position, a.n_entries, np.int32),
+                    values=_np_view(a.values, a.n_entries, np.float32),
+                    oc_order=_np_view(a.oc_order, a.n_slots, np.int32), stages=int(a.stages), tile_ic=int(a.tile_ic),
+                    nnz=int(a.nnz))
+
+    def launch(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0):
+        """Asynchronous conv on raw device pointers (NCHW in, NCHW out)."""
+        _check(_lib.tetris_spconv2d_launch(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h, img_w,
+                                           stride, padding, C.byref(tile) if tile is not None else None,
+                                           C.c_void_p(stream)))
+
+    def time(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0, warm=30, repeat=100):
+        ms = C.c_float()
+        _check(_lib.tetris_spconv2d_time(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h, img_w,
+                                         stride, padding, C.byref(tile) if tile is not None else None,
+                                         C.c_void_p(stream), warm, repeat, C.byref(ms)))
+        return float(ms.value)
+
+    def close(self):
+        if getattr(self, "_h", None) and _lib is not None:
+            _lib.tetris_g950_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+
+def tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding):
+    t = Tile()
+    _check(_lib.tetris_tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
+                                   C.byref(t)))
+    return t
+
+
+def SparseConv2d(input, offsets, stage_len, oc_permutation, position, values, output, batch_size, img_h, img_w,
+                 in_channel, out_channel, kernel_size, stride, padding, stream=0):
+    """The reference launcher's call shape on raw device pointers of a live SparseFilter."""
+    _check(_lib.tetris_spconv2d_launch_spf(C.c_void_p(input), C.c_void_p(offsets), C.c_void_p(stage_len),
+                                           C.c_void_p(oc_permutation), C.c_void_p(position), C.c_void_p(values),
+                                           C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel,
+                                           kernel_size, stride, padding, C.c_void_p(stream)))
+
+
+def _host_entry(fn, h_input, h_filter, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
+                stream, layout, apply_reorder):
+    x = np.ascontiguousarray(h_input, np.float32)
+    w = np.ascontiguousarray(h_filter, np.float32)
+    out = np.empty((batch_size, out_channel, out_extent(img_h, padding, kernel_size, stride),
+                    out_extent(img_w, padding, kernel_size, stride)), np.float32)
+    ms = C.c_float()
+    _check(fn(x, w, out, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
+              C.c_void_p(stream), layout.encode(), int(apply_reorder), C.byref(ms)))
+    return out, float(ms.value)
+
+
+def CudaSparseConv2d(h_input, h_filter, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
+                     padding, stream=0, layout="NHWC", apply_reorder=True):
+    """-> (h_output NCHW, mean ms per launch)."""
+    return _host_entry(_lib.tetris_spconv2d_host, h_input, h_filter, batch_size, img_h, img_w, in_channel,
+                       out_channel, kernel_size, stride, padding, stream, layout, apply_reorder)
+
+
+def SparseConv2d_SPF(h_input, h_filter, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
+                     padding, stream=0, layout="NHWC", apply_reorder=True):
+    return _host_entry(_lib.tetris_spconv2d_spf_host, h_input, h_filter, batch_size, img_h, img_w, in_channel,
+                       out_channel, kernel_size, stride, padding, stream, layout, apply_reorder)
+
+
+def ReadConfigAndDataFromFile(weight_file):
+    """-> (dict H W IC OC KS PAD STRIDE GROUPS, filter OIHW, nnz); raises TetrisError(EIO) if unreadable."""
+    hdr = (C.c_int32 * 8)()
+    ptr = C.POINTER(C.c_float)()
+    nnz = C.c_int64()
+    _check(_lib.tetris_read_weight_file(weight_file.encode(), hdr, C.byref(ptr), C.byref(nnz)))
+    h = dict(zip(("H", "W", "IC", "OC", "KS", "PAD", "STRIDE", "GROUPS"), [int(v) for v in hdr]))
+    n = h["OC"] * h["IC"] * h["KS"] * h["KS"]
+    w = np.ctypeslib.as_array(ptr, shape=(n,)).copy().reshape(h["OC"], h["IC"], h["KS"], h["KS"])
+    _lib.tetris_free(ptr)
+    return h, w, int(nnz.value)
+
+
+def FloatEqual(x, y):
+    return bool(_lib.tetris_float_equal(x, y))
+
+
+def TensorEqual(x, y):
+    x = np.ascontiguousarray(x, np.float32).ravel()
+    y = np.ascontiguousarray(y, np.float32).ravel()
+    return int(_lib.tetris_tensor_first_mismatch(x, y, x.size)) == -1
