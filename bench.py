@@ -38,6 +38,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
     ap.add_argument("--layer-repeat", type=int, default=30, help="timed launches per layer for the per-layer table")
+    ap.add_argument("--tile", choices=("autotune", "select"), default="autotune",
+                    help="autotune: time the selector's best candidates per layer during set-up (what the reference's "
+                         "driver does with its 185-entry table); select: take the selector's first choice unmeasured")
+    ap.add_argument("--candidates", type=int, default=24)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU (no collectives or sharding are part of the path); "
@@ -59,9 +63,12 @@ def main():
     t_pack = 0.0
     for L in layers:
         w = W.make_weights(L)
-        tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+        if args.tile == "autotune":
+            tile, _ = T.tile_autotune(w, N, L.H, L.W, L.stride, L.pad, args.candidates)
+        else:
+            tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
         t0 = time.perf_counter()
-        pk = T.G950Filter(w, tile.tile_ic)
+        pk = T.G950Filter.for_tile(w, tile)
         torch.cuda.synchronize()
         t_pack += time.perf_counter() - t0
         x = torch.from_numpy(W.make_activations(L, N)).to(dev)
@@ -141,7 +148,7 @@ def main():
         for L in sample_layers:
             w = W.make_weights(L)
             x1 = W.make_activations(L, 1)
-            pk = O.G950Pack(w, 32)
+            pk = O.G950Pack(w, 32, 8)
             t0 = time.perf_counter()
             pk.conv(x1, L.stride, L.pad, threads=threads)
             t_cpu += time.perf_counter() - t0
@@ -174,6 +181,7 @@ def main():
         "sparse_gflops": round(fl_sparse / (ms_per_step * 1e-3) / 1e9, 1),
         "sum_layer_us": round(t_layers * 1e6, 1),
         "pack_ms_total": round(t_pack * 1e3, 2),
+        "tile_selection": args.tile,
         "roofline": roofline,
         "cpu_baseline": cpu,
         "check": check,

@@ -63,9 +63,12 @@ int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* out);
 
 /* ------------------------------------------------------------------------------------------------
  * Weight preprocessing, gfx950 layout: a device pass (count, scan, scatter) over the dense OIHW
- * filter that writes, per (output-channel slot, input-channel stage), the non-zero entries in
- * (channel, row, column) order, padded with zero entries to a multiple of 8 so that a wave fetches
- * eight (offset, value) pairs with one 64-byte scalar load.
+ * filter.  Output-channel slots are taken `oc_per_wave` at a time (one group per wave of the conv
+ * kernel); per (group, input-channel stage) it writes ONE stream with the group's non-zero entries,
+ * position by position (channel, row, column ascending; slots ascending inside a position), padded
+ * with zero entries to a multiple of 8 so that a wave fetches eight (position, value) pairs with one
+ * 64-byte scalar load.  The position word is the reference's s | r<<3 | (ic % tile_ic)<<6
+ * (Tetris/spconv2d_utils.h:91) with the slot's index inside its group in bits 24..31.
  * No reference counterpart for the layout; it plays the role of the SparseFilter constructor for the
  * HIP kernel.  `oc_order` (may be NULL = identity) lists, slot by slot, which output channel a slot
  * computes -- pass a tetris_spf's oc_permutation to keep the reference's channel regrouping.
@@ -73,19 +76,20 @@ int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* out);
 typedef struct tetris_g950 tetris_g950;
 
 int tetris_g950_create(const float* h_filter_oihw, int in_channel, int out_channel, int kernel_size, int tile_ic,
-                       const int32_t* oc_order, void* stream, tetris_g950** out);
+                       int oc_per_wave, const int32_t* oc_order, void* stream, tetris_g950** out);
 /* Same, from a filter already resident in device memory. */
 int tetris_g950_create_device(const float* d_filter_oihw, int in_channel, int out_channel, int kernel_size,
-                              int tile_ic, const int32_t* oc_order, void* stream, tetris_g950** out);
+                              int tile_ic, int oc_per_wave, const int32_t* oc_order, void* stream,
+                              tetris_g950** out);
 void tetris_g950_destroy(tetris_g950* p);
 
 typedef struct tetris_g950_arrays {
-  const int32_t* seg_offsets; int64_t n_seg_offsets; /* [slots*stages+1], entry index, multiples of 8 */
-  const int32_t* seg_nnz;     int64_t n_seg_nnz;     /* [slots*stages], real entries in the segment    */
-  const int32_t* position;    int64_t n_entries;     /* s | r<<3 | (ic % tile_ic)<<6, 0 for padding    */
-  const float*   values;                             /* 0.0f for padding                               */
-  const int32_t* oc_order;    int64_t n_slots;       /* output channel of each slot                    */
-  int32_t stages, tile_ic;
+  const int32_t* grp_offsets; int64_t n_grp_offsets; /* [groups*stages+1], entry index, multiples of 8  */
+  const int32_t* grp_nnz;     int64_t n_grp_nnz;     /* [groups*stages], real entries in the stream     */
+  const int32_t* position;    int64_t n_entries;     /* s | r<<3 | (ic % tile_ic)<<6 | slot-in-group<<24 */
+  const float*   values;                             /* 0.0f for padding                                */
+  const int32_t* oc_order;    int64_t n_slots;       /* output channel of each slot, -1 for padding     */
+  int32_t stages, tile_ic, oc_per_wave;
   int64_t nnz;
 } tetris_g950_arrays;
 
@@ -94,19 +98,28 @@ int tetris_g950_host_arrays(tetris_g950* p, tetris_g950_arrays* out);
 
 /* ------------------------------------------------------------------------------------------------
  * Tile shape of the conv kernel.  Replaces the template arguments <TILE_IC, TILE_H, TILE_W> of the
- * reference launcher and its exhaustive table (Tetris/spconv2d.cc:90-329).  A zeroed struct means
- * "choose for me".
+ * reference launcher and its exhaustive table (Tetris/spconv2d.cc:90-329).  On launch, tile_ic and
+ * oc_per_wave must be the ones the pack was created with; a NULL tile means "choose for me" and needs
+ * a pack created with the tile_ic and oc_per_wave that tetris_tile_select returns for the shape.
  * ---------------------------------------------------------------------------------------------- */
 typedef struct tetris_tile {
-  int32_t lanes_w;     /* lanes across a tile row; the tile is 4*lanes_w output columns wide      */
+  int32_t lanes_w;     /* active lanes across a tile row (1..62); the tile is 4*lanes_w columns wide */
   int32_t quads;       /* 4-pixel groups per lane (1, 2 or 4)                                      */
-  int32_t oc_per_wave; /* output channels a wave accumulates at once (4, 8 or 16)                  */
-  int32_t waves;       /* waves per workgroup (1..16); workgroup computes waves*oc_per_wave channels */
-  int32_t tile_ic;     /* input channels staged in LDS at a time (informative on launch: the pack's) */
+  int32_t oc_per_wave; /* output channels a wave accumulates at once; oc_per_wave*4*quads <= 128   */
+  int32_t waves;       /* waves per workgroup (1, 2, 4 or 8); it computes waves*oc_per_wave channels */
+  int32_t tile_ic;     /* input channels staged in LDS at a time                                   */
 } tetris_tile;
 
 int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_channel, int kernel_size, int stride,
                        int padding, tetris_tile* out);
+
+/* Measured selection, the counterpart of GetTetrisSparseConv2dTime (Tetris/spconv2d.cc:72-329): packs the filter
+ * for the `max_candidates` (0 = 24) tile shapes the model of tetris_tile_select ranks best, times each on the
+ * device with the real weights (1 warm-up + 3 launches on zero-filled input) and returns the fastest and its
+ * milliseconds per launch.  Allocates and frees its own device buffers; synchronises `stream`. */
+int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int img_w, int in_channel, int out_channel,
+                         int kernel_size, int stride, int padding, int max_candidates, void* stream,
+                         tetris_tile* out, float* ms_out);
 
 /* ------------------------------------------------------------------------------------------------
  * Conv launch on device tensors.  Replaces: SparseConv2d<float,int,int,KS,STRIDE,TILE_IC,TILE_H,TILE_W>

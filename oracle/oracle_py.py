@@ -58,11 +58,11 @@ if _lib is not None:
         getattr(_lib, "orc_pack_" + _n).restype = C.POINTER(_t)
     _lib.orc_host_spconv2d.argtypes = [C.c_void_p, _f32p, _f32p] + [C.c_int] * 6
     _lib.orc_host_reorder_spconv2d.argtypes = [C.c_void_p, _f32p, _f32p] + [C.c_int] * 6
-    _lib.orc_g950_pack.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    _lib.orc_g950_pack.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
     _lib.orc_g950_pack.restype = C.c_void_p
     _lib.orc_g950_free.argtypes = [C.c_void_p]
     _lib.orc_g950_sizes.argtypes = [C.c_void_p, C.POINTER(C.c_int64)]
-    for _n, _t in (("seg_off", C.c_int32), ("seg_nnz", C.c_int32), ("position", C.c_int32), ("values", C.c_float),
+    for _n, _t in (("grp_off", C.c_int32), ("grp_nnz", C.c_int32), ("position", C.c_int32), ("values", C.c_float),
                    ("order", C.c_int32)):
         getattr(_lib, "orc_g950_" + _n).argtypes = [C.c_void_p]
         getattr(_lib, "orc_g950_" + _n).restype = C.POINTER(_t)
@@ -201,12 +201,12 @@ class SpfPack:
 class G950Pack:
     """Result of orc_g950_pack: the layout the HIP kernel consumes, built on the CPU."""
 
-    def __init__(self, w, tile_ic, order=None):
+    def __init__(self, w, tile_ic, oc_per_wave, order=None):
         w = np.ascontiguousarray(w, np.float32)
         self.K, self.C, self.ks, _ = w.shape
-        self.tile_ic = tile_ic
+        self.tile_ic, self.oc_per_wave = tile_ic, oc_per_wave
         o = None if order is None else np.ascontiguousarray(order, np.int32)
-        self._h = _lib.orc_g950_pack(w, self.C, self.K, self.ks, tile_ic,
+        self._h = _lib.orc_g950_pack(w, self.C, self.K, self.ks, tile_ic, oc_per_wave,
                                      None if o is None else o.ctypes.data_as(C.c_void_p))
         n = (C.c_int64 * 5)()
         _lib.orc_g950_sizes(self._h, n)
@@ -217,8 +217,8 @@ class G950Pack:
                 return np.zeros(0, dt)
             return np.ctypeslib.as_array(getattr(_lib, "orc_g950_" + name)(self._h), shape=(cnt,)).copy()
 
-        self.seg_off = grab("seg_off", n[0], np.int32)
-        self.seg_nnz = grab("seg_nnz", n[1], np.int32)
+        self.grp_off = grab("grp_off", n[0], np.int32)
+        self.grp_nnz = grab("grp_nnz", n[1], np.int32)
         self.position = grab("position", n[2], np.int32)
         self.values = grab("values", n[2], np.float32)
         self.order = grab("order", n[3], np.int32)

@@ -499,84 +499,98 @@ void orc_host_reorder_spconv2d(const OrcPack* p, const float* input, float* outp
 
 // ---- gfx950 layout (defined by this project; no reference counterpart) --------------------------
 // Slots = K rounded up to a multiple of 128; slot i computes output channel order[i] (identity when
-// order == NULL), padding slots hold -1 and empty runs.  Per (slot, stage): the non-zero weights of
-// channels [stage*tile_ic, ...) in (channel, row, column) order -- the scan order of
-// spconv2d_utils.h:85-94 -- with the reference's position word (:91), then (0, 0.0f) entries up to a
-// multiple of 8.  seg_off is the running sum of the padded run lengths.
+// order == NULL), padding slots hold -1.  Slots are taken G at a time (one group per wave of the HIP
+// kernel).  Per (group, stage) one stream: for every position of the stage in (channel, row, column)
+// order -- the scan order of spconv2d_utils.h:85-94 -- and every slot l of the group in ascending
+// order, the non-zero weight with the position word of spconv2d_utils.h:91 plus l << 24; then
+// (0, 0.0f) entries up to a multiple of 8.  grp_off is the running sum of the padded stream lengths.
 struct OrcG950 {
-  int C = 0, K = 0, ks = 0, tile_ic = 0, stages = 0, slots = 0;
-  std::vector<int32_t> seg_off, seg_nnz, position, order;
+  int C = 0, K = 0, ks = 0, tile_ic = 0, stages = 0, slots = 0, G = 0, groups = 0;
+  std::vector<int32_t> grp_off, grp_nnz, position, order;
   std::vector<float> values;
 };
 
-OrcG950* orc_g950_pack(const float* filter, int C, int K, int ks, int tile_ic, const int32_t* order) {
+OrcG950* orc_g950_pack(const float* filter, int C, int K, int ks, int tile_ic, int G, const int32_t* order) {
   OrcG950* P = new OrcG950;
-  P->C = C; P->K = K; P->ks = ks; P->tile_ic = tile_ic;
+  P->C = C; P->K = K; P->ks = ks; P->tile_ic = tile_ic; P->G = G;
   P->stages = (C - 1) / tile_ic + 1;
   P->slots = (K + 127) / 128 * 128;
+  P->groups = P->slots / G;
   P->order.assign(P->slots, -1);
   for (int i = 0; i < K; ++i) P->order[i] = order ? order[i] : i;
-  P->seg_off.push_back(0);
+  P->grp_off.push_back(0);
   const int kk = ks * ks;
-  for (int slot = 0; slot < P->slots; ++slot)
+  for (int grp = 0; grp < P->groups; ++grp)
     for (int st = 0; st < P->stages; ++st) {
       int n = 0;
-      const int oc = P->order[slot];
-      if (oc >= 0)
-        for (int j = st * tile_ic; j < std::min((st + 1) * tile_ic, C); ++j)
-          for (int r = 0; r < ks; ++r)
-            for (int s = 0; s < ks; ++s) {
+      for (int j = st * tile_ic; j < std::min((st + 1) * tile_ic, C); ++j)
+        for (int r = 0; r < ks; ++r)
+          for (int s = 0; s < ks; ++s)
+            for (int l = 0; l < G; ++l) {
+              const int oc = P->order[grp * G + l];
+              if (oc < 0) continue;
               const float v = filter[(size_t)oc * C * kk + (size_t)j * kk + r * ks + s];
               if (v != 0.f) {
-                P->position.push_back(make_pos(s, r, j % tile_ic));
+                P->position.push_back(make_pos(s, r, j % tile_ic) + (l << 24));
                 P->values.push_back(v);
                 ++n;
               }
             }
-      P->seg_nnz.push_back(n);
+      P->grp_nnz.push_back(n);
       for (int i = n; i % 8 != 0; ++i) {
         P->position.push_back(0);
         P->values.push_back(0.0f);
       }
-      P->seg_off.push_back((int32_t)P->position.size());
+      P->grp_off.push_back((int32_t)P->position.size());
     }
   return P;
 }
 void orc_g950_free(OrcG950* p) { delete p; }
 void orc_g950_sizes(const OrcG950* p, int64_t* n) {
-  n[0] = (int64_t)p->seg_off.size(); n[1] = (int64_t)p->seg_nnz.size(); n[2] = (int64_t)p->position.size();
+  n[0] = (int64_t)p->grp_off.size(); n[1] = (int64_t)p->grp_nnz.size(); n[2] = (int64_t)p->position.size();
   n[3] = p->slots; n[4] = p->stages;
 }
-const int32_t* orc_g950_seg_off(const OrcG950* p) { return p->seg_off.data(); }
-const int32_t* orc_g950_seg_nnz(const OrcG950* p) { return p->seg_nnz.data(); }
+const int32_t* orc_g950_grp_off(const OrcG950* p) { return p->grp_off.data(); }
+const int32_t* orc_g950_grp_nnz(const OrcG950* p) { return p->grp_nnz.data(); }
 const int32_t* orc_g950_position(const OrcG950* p) { return p->position.data(); }
 const float* orc_g950_values(const OrcG950* p) { return p->values.data(); }
 const int32_t* orc_g950_order(const OrcG950* p) { return p->order.data(); }
 
-// Convolution straight from the gfx950 arrays, accumulating in run order (stage by stage, entry by
-// entry, padding entries included) -- the order the HIP kernel adds in, without its fused multiply-add.
+// Convolution straight from the gfx950 arrays: every output accumulates its slot's entries in stream
+// order (stage by stage) -- the order the HIP kernel adds in, without its fused multiply-add.
 void orc_g950_conv(const OrcG950* p, const float* input, float* output, int N, int H, int W, int pad, int stride,
                    int threads) {
-  const int C = p->C, K = p->K, ks = p->ks, S = p->stages, T = p->tile_ic;
+  const int C = p->C, K = p->K, ks = p->ks, S = p->stages, T = p->tile_ic, G = p->G;
   const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
 #pragma omp parallel for collapse(2) schedule(dynamic) num_threads(threads > 0 ? threads : 1)
   for (int n = 0; n < N; ++n)
-    for (int slot = 0; slot < p->slots; ++slot) {
-      const int oc = p->order[slot];
-      if (oc < 0) continue;
-      for (int h = 0; h < OH; ++h)
-        for (int w = 0; w < OW; ++w) {
-          float sum = 0;
-          for (int st = 0; st < S; ++st)
-            for (int e = p->seg_off[slot * S + st]; e < p->seg_off[slot * S + st + 1]; ++e) {
-              const int pos = p->position[e];
-              const int y = pos & 7, x = (pos >> kBitS) & 7, ic = (pos >> (kBitS + kBitR)) + st * T;
-              const int ih = h * stride + x, iw = w * stride + y;
-              if (ih < pad || ih >= H + pad || iw < pad || iw >= W + pad) continue;
-              sum += input[(((size_t)n * C + ic) * H + (ih - pad)) * W + (iw - pad)] * p->values[e];
+    for (int grp = 0; grp < p->groups; ++grp) {
+      std::vector<float> acc((size_t)G * OH * OW, 0.f);
+      for (int st = 0; st < S; ++st)
+        for (int e = p->grp_off[grp * S + st]; e < p->grp_off[grp * S + st + 1]; ++e) {
+          const int pos = p->position[e];
+          const float v = p->values[e];
+          if (v == 0.f) continue;  // padding
+          const int y = pos & 7, x = (pos >> kBitS) & 7, ic = ((pos >> (kBitS + kBitR)) & 0x3ffff) + st * T;
+          const int l = (pos >> 24) & 0xff;
+          const float* img = &input[((size_t)n * C + ic) * H * W];
+          float* a = &acc[(size_t)l * OH * OW];
+          for (int h = 0; h < OH; ++h) {
+            const int ih = h * stride + x - pad;
+            if (ih < 0 || ih >= H) continue;
+            for (int w = 0; w < OW; ++w) {
+              const int iw = w * stride + y - pad;
+              if (iw < 0 || iw >= W) continue;
+              a[h * OW + w] += img[(size_t)ih * W + iw] * v;
             }
-          output[(((size_t)n * K + oc) * OH + h) * OW + w] = sum;
+          }
         }
+      for (int l = 0; l < G; ++l) {
+        const int oc = p->order[grp * G + l];
+        if (oc < 0) continue;
+        std::copy(acc.begin() + (size_t)l * OH * OW, acc.begin() + (size_t)(l + 1) * OH * OW,
+                  &output[((size_t)n * K + oc) * OH * OW]);
+      }
     }
 }
 

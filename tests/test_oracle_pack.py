@@ -151,3 +151,43 @@ def test_host_decoders_reproduce_dense_conv(oracle, shape):
         got = oracle.SpfPack(w, T, True, vec == 4, bool(bank), bool(reoc)).conv(x, stride, pad)
         np.testing.assert_allclose(got, dense, rtol=1e-5, atol=1e-5)
         assert oracle.tensor_first_mismatch(got, dense) == -1  # the reference's own tolerance predicate
+
+
+@pytest.mark.parametrize("shape", [(2, 20, 9, 11, 40, 3, 1, 1, 8, 8), (1, 48, 8, 8, 64, 1, 1, 0, 32, 16),
+                                   (1, 7, 13, 13, 33, 3, 2, 1, 4, 32), (2, 3, 17, 17, 16, 7, 2, 3, 3, 4),
+                                   (1, 70, 6, 6, 130, 1, 2, 0, 16, 8)])
+def test_gfx950_stream_layout(oracle, shape):
+    """The layout the HIP kernel consumes, as the oracle defines it: structure, content and convolution."""
+    n, c, h, w_, k, ks, stride, pad, T, G = shape
+    rng = np.random.default_rng(sum(shape))
+    w = sparse_filter(rng, k, c, ks, 0.8)
+    x = relu_like(rng, (n, c, h, w_))
+    order = rng.permutation(k).astype(np.int32)
+    for perm in (None, order):
+        p = oracle.G950Pack(w, T, G, perm)
+        S = (c - 1) // T + 1
+        assert p.slots == -(-k // 128) * 128 and p.stages == S
+        groups = p.slots // G
+        assert len(p.grp_off) == groups * S + 1 and p.grp_off[0] == 0
+        d = np.diff(p.grp_off)
+        assert (d % 8 == 0).all() and np.array_equal(-(-p.grp_nnz // 8) * 8, d)
+        assert int(p.grp_nnz.sum()) == int((w != 0).sum())
+        exp_order = np.full(p.slots, -1, np.int32)
+        exp_order[:k] = np.arange(k) if perm is None else perm
+        assert np.array_equal(p.order, exp_order)
+        got = Counter()
+        for grp in range(groups):
+            for st in range(S):
+                b, nn = int(p.grp_off[grp * S + st]), int(p.grp_nnz[grp * S + st])
+                pos, val = p.position[b:b + nn], p.values[b:b + nn]
+                key = (pos & 0xFFFFFF).astype(np.int64) * 256 + (pos >> 24)
+                assert (np.diff(key) > 0).all()  # position-major, slots ascending inside a position
+                assert (p.position[b + nn:p.grp_off[grp * S + st + 1]] == 0).all()
+                assert (p.values[b + nn:p.grp_off[grp * S + st + 1]] == 0).all()
+                for q, v in zip(pos, val):
+                    q = int(q)
+                    oc = int(exp_order[grp * G + (q >> 24)])
+                    got[(oc, ((q >> 6) & 0x3FFFF) + st * T, (q >> 3) & 7, q & 7, v.tobytes())] += 1
+        assert got == filter_nonzeros(w)
+        np.testing.assert_allclose(p.conv(x, stride, pad, threads=2), oracle.host_conv2d(x, w, stride, pad), rtol=1e-5,
+                                   atol=1e-5)

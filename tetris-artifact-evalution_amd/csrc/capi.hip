@@ -41,20 +41,42 @@ int upload(const std::vector<T>& v, T** d) {
 int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
                const tetris_tile* tile, hipStream_t stream) {
   if (!p || !d_in || !d_out) return fail(TETRIS_EINVAL, "null argument");
-  tetris_tile t{};
-  if (tile && tile->lanes_w > 0) {
-    t = *tile;
-  } else {
-    int rc = choose_tile(N, H, W, p->C, p->K, p->ks, stride, pad, &t);
-    if (rc) return rc;
+  const bool given = tile && tile->lanes_w > 0;
+  Plan plan;
+  bool found = false;
+  if (given) {
+    const int key[10] = {N, H, W, stride, pad, tile->lanes_w, tile->quads, tile->oc_per_wave, tile->waves, tile->tile_ic};
+    std::lock_guard<std::mutex> lock(p->mu);
+    for (size_t i = p->plans.size(); i-- > 0;)
+      if (memcmp(p->plans[i].key, key, sizeof key) == 0) {
+        plan = p->plans[i];
+        found = true;
+        break;
+      }
   }
-  Geom g;
-  int rc = make_geom(p, N, H, W, stride, pad, t, &g);
-  if (rc) return rc;
-  const int2* entries = nullptr;
-  rc = g950_bind(p, g, stream, &entries);
-  if (rc) return rc;
-  return launch_conv(g, t, d_in, d_out, entries, p->d_seg_off, p->d_oc_order, stream);
+  if (!found) {
+    tetris_tile t{};
+    if (given) {
+      t = *tile;
+    } else {
+      int rc = choose_tile(N, H, W, p->C, p->K, p->ks, stride, pad, &t);
+      if (rc) return rc;
+    }
+    if (t.tile_ic != p->tile_ic || t.oc_per_wave != p->g)
+      return fail(TETRIS_EINVAL, "tile (tile_ic=%d, oc_per_wave=%d) does not match the pack (tile_ic=%d, oc_per_wave=%d)",
+                  t.tile_ic, t.oc_per_wave, p->tile_ic, p->g);
+    int rc = make_geom(p, N, H, W, stride, pad, t, &plan.geom);
+    if (rc) return rc;
+    rc = g950_bind(p, plan.geom, stream, &plan.entries);
+    if (rc) return rc;
+    const int key[10] = {N, H, W, stride, pad, t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic};
+    memcpy(plan.key, key, sizeof key);
+    if (given) {
+      std::lock_guard<std::mutex> lock(p->mu);
+      if (p->plans.size() < 64) p->plans.push_back(plan);
+    }
+  }
+  return launch_conv(plan.geom, d_in, d_out, plan.entries, p->d_grp_off, p->d_oc_order, stream);
 }
 
 int time_launches(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
@@ -104,7 +126,8 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
     order = spf->oc_permutation;
   }
   tetris_g950* pack = nullptr;
-  rc = tetris_g950_create(h_filter, C, K, ks, tile.tile_ic, apply_reorder ? order.data() : nullptr, stream, &pack);
+  rc = tetris_g950_create(h_filter, C, K, ks, tile.tile_ic, tile.oc_per_wave, apply_reorder ? order.data() : nullptr,
+                          stream, &pack);
   float *d_in = nullptr, *d_out = nullptr;
   const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
   auto done = [&](int code) {
@@ -169,14 +192,16 @@ static int spf_ensure_device(tetris_spf* f) {
 }
 
 // The kernel's own pack of this filter for `tile_ic` staged input channels, in the same slot order.
-static int spf_kernel_pack(tetris_spf* f, int tile_ic, hipStream_t stream, tetris_g950** out) {
+static int spf_kernel_pack(tetris_spf* f, int tile_ic, int oc_per_wave, hipStream_t stream, tetris_g950** out) {
   std::lock_guard<std::mutex> lock(f->mu);
-  auto it = f->kernel_packs.find(tile_ic);
+  const std::pair<int, int> key(tile_ic, oc_per_wave);
+  auto it = f->kernel_packs.find(key);
   if (it == f->kernel_packs.end()) {
     tetris_g950* p = nullptr;
-    int rc = tetris_g950_create(f->filter.data(), f->C, f->K, f->ks, tile_ic, f->oc_permutation.data(), stream, &p);
+    int rc = tetris_g950_create(f->filter.data(), f->C, f->K, f->ks, tile_ic, oc_per_wave, f->oc_permutation.data(),
+                                stream, &p);
     if (rc) return rc;
-    it = f->kernel_packs.emplace(tile_ic, p).first;
+    it = f->kernel_packs.emplace(key, p).first;
   }
   *out = it->second;
   return TETRIS_OK;
@@ -242,6 +267,67 @@ int tetris_tile_select(int N, int H, int W, int C, int K, int ks, int stride, in
   return choose_tile(N, H, W, C, K, ks, stride, pad, out);
 }
 
+int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int K, int ks, int stride, int pad,
+                         int max_candidates, void* stream_, tetris_tile* out, float* ms_out) {
+  if (!h_filter || !out) return fail(TETRIS_EINVAL, "null argument");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  std::vector<tetris_tile> ranked;
+  int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked);
+  if (rc) return rc;
+  if (max_candidates <= 0) max_candidates = 24;
+  const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
+  const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
+  const size_t f_bytes = sizeof(float) * (size_t)C * K * ks * ks;
+  float *d_in = nullptr, *d_out = nullptr, *d_f = nullptr;
+  std::map<std::pair<int, int>, tetris_g950*> packs;
+  auto done = [&](int code) {
+    for (auto& kv : packs) tetris_g950_destroy(kv.second);
+    if (d_in) (void)hipFree(d_in);
+    if (d_out) (void)hipFree(d_out);
+    if (d_f) (void)hipFree(d_f);
+    return code;
+  };
+#define HIPA(call)                                                                                          \
+  do {                                                                                                      \
+    hipError_t e_ = (call);                                                                                 \
+    if (e_ != hipSuccess)                                                                                   \
+      return done(fail(TETRIS_EHIP, "%s failed at %s:%d: %s", #call, __FILE__, __LINE__, hipGetErrorString(e_))); \
+  } while (0)
+  HIPA(hipMalloc(&d_in, in_bytes));
+  HIPA(hipMalloc(&d_out, out_bytes));
+  HIPA(hipMalloc(&d_f, f_bytes));
+  HIPA(hipMemsetAsync(d_in, 0, in_bytes, stream));  // timing does not depend on the values
+  HIPA(hipMemcpyAsync(d_f, h_filter, f_bytes, hipMemcpyHostToDevice, stream));
+#undef HIPA
+  float best_ms = 1e30f;
+  tetris_tile best = ranked[0];
+  int tried = 0;
+  for (const tetris_tile& t : ranked) {
+    if (tried >= max_candidates) break;
+    const std::pair<int, int> key(t.tile_ic, t.oc_per_wave);
+    auto it = packs.find(key);
+    if (it == packs.end()) {
+      tetris_g950* p = nullptr;
+      rc = tetris_g950_create_device(d_f, C, K, ks, t.tile_ic, t.oc_per_wave, nullptr, stream, &p);
+      if (rc) return done(rc);
+      it = packs.emplace(key, p).first;
+    }
+    float ms = 0;
+    rc = time_launches(it->second, d_in, d_out, N, H, W, stride, pad, &t, stream, 1, 3, &ms);
+    if (rc == TETRIS_EINVAL) continue;  // the model ranks shapes make_geom may still refuse
+    if (rc) return done(rc);
+    ++tried;
+    if (ms < best_ms) {
+      best_ms = ms;
+      best = t;
+    }
+  }
+  if (tried == 0) return done(fail(TETRIS_EINVAL, "no tile shape could be launched for this layer"));
+  *out = best;
+  if (ms_out) *ms_out = best_ms;
+  return done(TETRIS_OK);
+}
+
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
                            const tetris_tile* tile, void* stream) {
   return run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, static_cast<hipStream_t>(stream));
@@ -265,7 +351,7 @@ int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, cons
   int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &t);
   if (rc) return rc;
   tetris_g950* pack = nullptr;
-  rc = spf_kernel_pack(f, t.tile_ic, static_cast<hipStream_t>(stream), &pack);
+  rc = spf_kernel_pack(f, t.tile_ic, t.oc_per_wave, static_cast<hipStream_t>(stream), &pack);
   if (rc) return rc;
   return run_launch(pack, d_in, d_out, N, H, W, stride, pad, &t, static_cast<hipStream_t>(stream));
 }

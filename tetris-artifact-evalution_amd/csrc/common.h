@@ -27,74 +27,104 @@ int fail(int code, const char* fmt, ...);  // records the message for tetris_las
                             hipGetErrorString(e_));                                                \
   } while (0)
 
-constexpr int kBatch = 8;        // entries per 64-byte scalar fetch; segments are padded to this
-constexpr int kWave = 64;
+constexpr int kBatch = 8;        // entries per 64-byte scalar fetch; every stream is padded to this
 constexpr int kRefLanes = 32;    // the reference layout's lane count (Tetris/spconv2d_utils.h:15)
 constexpr int kMaxKs = 7;        // 3-bit row/column fields of the position word
+constexpr int kSlotPad = 128;    // output-channel slots are padded to a multiple of this
+constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (all regions)
+constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4 * quads
+constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
 
 inline int out_extent(int in, int pad, int ks, int stride) { return (in + 2 * pad - ks) / stride + 1; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // ---- kernel geometry --------------------------------------------------------------------------
-// One workgroup computes, for `nb` images, a `thi` x (4*lw) patch of output pixels and
-// waves*G output-channel slots.  A lane owns `NQ` quads; quad q of lane (ly, lx) is the four pixels
-// (virtual row ly + q*lh, columns lx + j*lw, j = 0..3).  Virtual row v is row v % thi of image v / thi.
+// Output pixels are cut into *units* of up to 64 quads: a unit is `lh` virtual rows by 4*lw columns, lane
+// (ly, lx) = (lane / lr, lane % lr) owning the four pixels (virtual row ly, columns lx + j*lw, j = 0..3);
+// lanes with lx >= lw or ly >= lh idle.  A virtual row v is row v % thi of image v / thi, so that small
+// feature maps fold several images into one unit.  A workgroup computes NQ consecutive units (one per
+// lane "quad") for waves * G output-channel slots.
 //
-// LDS holds, per image and staged input channel, `ih` input rows of `pitch` dwords.  A row stores the
-// columns regrouped so that the four inputs a quad needs for kernel column s sit in one aligned
-// 16-byte slot: with u = stride*lx + s, slot (u % stride, u / stride) holds input columns
-// u + stride*lw*j, j = 0..3.  Slots of one parity (u % stride) are contiguous (`par` dwords apart per
-// parity), so neighbouring lanes read neighbouring slots for every s and every stride.
+// Why lr (lanes per row) can exceed lw: a 16-byte-per-lane LDS read runs at the full 256 B/clk only when
+// every lane row starts, bank-wise, where the previous one ended, i.e. when the LDS distance between
+// consecutive lane rows is 4*lr dwords modulo 64 (measured on MI355X; any other distance halves the
+// rate).  A halo'd row holds lw + (ks-1)/stride slots, so the lanes of a row are spread over that many
+// lane positions and the pitch is chosen to meet the rule.
+//
+// LDS holds one region of kTileBytes / NQ bytes per unit: [image][staged channel][input row][pitch]
+// floats.  A row stores its columns regrouped so that the four inputs a quad needs for kernel column s
+// sit in one aligned 16-byte slot: with u = stride*lx + s, slot (u % stride, u / stride) holds input
+// columns u + stride*lw*j, j = 0..3.  Slots of one parity (u % stride) are contiguous, `par` dwords
+// per parity, so neighbouring lanes read neighbouring slots for every s and every stride.
 struct Geom {
   int N, C, H, W, K, OH, OW, ks, stride, pad;
   int tile_ic, stages;
-  int lw, lh, thi, nb;
-  int ng;          // 16-byte slots per parity per row
-  int pitch;       // dwords per LDS row (>= stride*ng*4)
-  int par;         // dwords between parity planes inside a row (= ng*4)
-  int ih;          // staged input rows per image
-  int plane;       // dwords per (image, channel) = ih*pitch
-  int img_stride;  // dwords per image = tile_ic*plane
-  int fill_slots;  // nb*ih*stride*ng: 16-byte slots to fill per staged channel
-  int tiles_w, tiles_h, tiles_n;
-  int kblocks;     // workgroups along the output-channel slots
-  int kb;          // slots per workgroup = waves*G
-  int slots;       // padded slot count of the pack
-  int lds_bytes;   // tile + fill table
+  int nq, g, waves;    // quads per lane, slots per wave, waves per workgroup
+  int lw, lr, lh, thi, nb; // active lanes per row, lane positions per row, lane rows, rows per image, images per unit
+  int ng;              // 16-byte slots per parity per row
+  int pitch;           // dwords per LDS row (>= stride*ng*4)
+  int par;             // dwords between parity planes inside a row (= ng*4)
+  int ih;              // staged input rows per image
+  int plane;           // dwords per (image, channel) = ih*pitch
+  int img_stride;      // dwords per image = tile_ic*plane
+  int region;          // bytes per region = kTileBytes / nq
+  int units_w, units_h, units_n, units;  // unit grid: columns, row blocks, image blocks, total
+  int ugroups;         // workgroups along the units = ceil(units / nq)
+  int kblocks;         // workgroups along the output-channel slots
+  int kb;              // slots per workgroup = waves*g
+  int slots;           // padded slot count of the pack
+  // input staging: a thread owns `spt` of the unit group's 16-byte slots and walks the staged channels
+  // `cg` at a time
+  int slots_per_unit;  // nb*ih*stride*ng
+  int fill_slots;      // nq*slots_per_unit
+  int spt, cg, fill_iters;
 };
 
-// Byte offset (inside one image's LDS tile) that the packed entry (ic_local, r, s) adds to a lane's base.
-inline int lds_entry_offset(const Geom& g, int ic_local, int r, int s) {
-  return 4 * (ic_local * g.plane + r * g.pitch + (s % g.stride) * g.par + (s / g.stride) * 4);
+// Byte offset that the packed entry (ic_local, r, s) adds to a lane's LDS base address.
+inline int lds_entry_offset(int plane, int pitch, int par, int stride, int ic_local, int r, int s) {
+  return 4 * (ic_local * plane + r * pitch + (s % stride) * par + (s / stride) * 4);
 }
 
-// ---- gfx950 pack ------------------------------------------------------------------------------
 struct BoundKey {
-  int plane, pitch, par, stride;
+  int plane, pitch, par, stride, nq;
   bool operator<(const BoundKey& o) const {
     if (plane != o.plane) return plane < o.plane;
     if (pitch != o.pitch) return pitch < o.pitch;
     if (par != o.par) return par < o.par;
-    return stride < o.stride;
+    if (stride != o.stride) return stride < o.stride;
+    return nq < o.nq;
   }
 };
 
 }  // namespace tetris
 
+namespace tetris {
+// A launch plan: everything run_launch derives from (input shape, tile) for one pack, kept for the next call.
+struct Plan {
+  int key[10];  // N, H, W, stride, pad, lanes_w, quads, oc_per_wave, waves, tile_ic
+  Geom geom;
+  const int2* entries;
+};
+}  // namespace tetris
+
+// gfx950 pack: per (wave group of G slots, input-channel stage) one stream of entries.
 struct tetris_g950 {
   int C = 0, K = 0, ks = 0, tile_ic = 0, stages = 0;
-  int slots = 0;            // K rounded up to a multiple of 128
+  int g = 0;                // slots per wave group
+  int slots = 0;            // K rounded up to a multiple of kSlotPad
+  int groups = 0;           // slots / g
   int64_t n_entries = 0, nnz = 0;
-  int32_t* d_seg_off = nullptr;   // [slots*stages+1]
-  int32_t* d_seg_nnz = nullptr;   // [slots*stages]
-  int32_t* d_position = nullptr;  // [n_entries]
+  int32_t* d_grp_off = nullptr;   // [groups*stages+1] entry index, multiples of 8
+  int32_t* d_grp_nnz = nullptr;   // [groups*stages]
+  int32_t* d_position = nullptr;  // [n_entries] s | r<<3 | ic_local<<6 | lane<<24
   float* d_values = nullptr;      // [n_entries]
   int32_t* d_oc_order = nullptr;  // [slots], -1 for padding slots
-  // (LDS byte offset, value) pairs for one tile geometry, made on first use
+  // (LDS byte offset | accumulator index << 24, value) pairs for one tile geometry, made on first use
   std::map<tetris::BoundKey, int2*> bound;
+  std::vector<tetris::Plan> plans;  // few per pack; searched linearly, most recent first
   std::mutex mu;
   // host mirrors, filled by tetris_g950_host_arrays
-  std::vector<int32_t> h_seg_off, h_seg_nnz, h_position, h_oc_order;
+  std::vector<int32_t> h_grp_off, h_grp_nnz, h_position, h_oc_order;
   std::vector<float> h_values;
 };
 
@@ -105,8 +135,8 @@ struct tetris_spf {
   std::vector<float> values;
   int32_t *d_offsets = nullptr, *d_stage_len = nullptr, *d_position = nullptr, *d_oc_permutation = nullptr;
   float* d_values = nullptr;
-  std::vector<float> filter;                   // dense copy the kernel's packs are made from
-  std::map<int, tetris_g950*> kernel_packs;    // by staged input channels, made at launch
+  std::vector<float> filter;                              // dense copy the kernel's packs are made from
+  std::map<std::pair<int, int>, tetris_g950*> kernel_packs;  // by (staged input channels, slots per wave)
   std::mutex mu;
 };
 
@@ -122,11 +152,12 @@ int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** en
 // tile_select.cpp
 int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile& t, Geom* g);
 int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t);
+// every tile shape the kernel can run for the layer, cheapest first by the selector's time model
+int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked);
 
 // spconv2d_kernel.hip
-int launch_conv(const Geom& g, const tetris_tile& t, const float* d_in, float* d_out, const int2* entries,
-                const int32_t* seg_off, const int32_t* oc_order, hipStream_t stream);
-size_t conv_lds_bytes(const Geom& g);
+int launch_conv(const Geom& g, const float* d_in, float* d_out, const int2* entries, const int32_t* grp_off,
+                const int32_t* oc_order, hipStream_t stream);
 
 }  // namespace tetris
 

@@ -1,50 +1,53 @@
-// gfx950 weight-preprocessing pass: dense OIHW fp32 filter -> per-(slot, stage) runs of non-zero
-// (position, value) entries, built on the device in three deterministic kernels (count, scan, scatter).
+// gfx950 weight-preprocessing pass: dense OIHW fp32 filter -> one stream of non-zero (position, value)
+// entries per (wave group of G output-channel slots, input-channel stage), built on the device in three
+// deterministic kernels (count, scan, scatter).
 //
 // Takes the place of the reference's host-side SparseFilter constructor (Tetris/spconv2d_utils.h:62-98,
 // :206-244) for the HIP kernel.  The position word keeps the reference encoding
-// s | r << 3 | (ic % tile_ic) << 6 (spconv2d_utils.h:91) and the zero test keeps `value != 0.f`, so -0.0
-// is dropped like the reference drops it.  What differs is the arrangement: the reference interleaves 32
-// lanes x 4 entries because its lanes are output channels; here every entry is wave-uniform, so a run
-// belongs to one output channel and is padded to a multiple of 8 entries (one 64-byte scalar fetch).
+// s | r << 3 | (ic % tile_ic) << 6 (spconv2d_utils.h:91) in its low 24 bits, and the zero test keeps
+// `value != 0.f`, so -0.0 is dropped like the reference drops it.  What differs is the arrangement: the
+// reference interleaves 32 lanes x 4 entries because its lanes are output channels; here every entry is
+// wave-uniform.  A stream lists the non-zeros of the group's G channels position by position (channel,
+// row, column ascending; within a position by slot), carries the slot's index inside the group in bits
+// 24..31, and is padded with zero entries to a multiple of 8 (one 64-byte scalar fetch).
 #include "common.h"
 
 namespace tetris {
 namespace {
 
-// one wave per (slot, stage): the stage's weights are cs*ks*ks consecutive floats
+// one wave per (group, stage); element i of the stage is (position i / G, slot i % G)
 __global__ __launch_bounds__(256) void count_kernel(const float* __restrict__ filter, const int32_t* __restrict__ oc_order,
-                                                    int32_t* __restrict__ seg_nnz, int32_t* __restrict__ seg_pad, int C,
-                                                    int ks, int tile_ic, int stages, int nseg) {
-  const int seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+                                                    int32_t* __restrict__ grp_nnz, int32_t* __restrict__ grp_pad, int C,
+                                                    int ks, int tile_ic, int stages, int G, int nstream) {
+  const int sid = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  if (seg >= nseg) return;
-  const int slot = seg / stages, st = seg - slot * stages;
-  const int oc = oc_order[slot];
+  if (sid >= nstream) return;
+  const int grp = sid / stages, st = sid - grp * stages;
+  const int kk = ks * ks;
+  const int c0 = st * tile_ic;
+  const int n = min(tile_ic, C - c0) * kk * G;
   int cnt = 0;
-  if (oc >= 0) {
-    const int kk = ks * ks;
-    const int c0 = st * tile_ic;
-    const int n = min(tile_ic, C - c0) * kk;
-    const float* src = filter + ((size_t)oc * C + c0) * kk;
-    for (int i = lane; i < n; i += 64) cnt += (src[i] != 0.f) ? 1 : 0;
-    for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
+  for (int i = lane; i < n; i += 64) {
+    const int p = i / G, l = i - p * G;
+    const int oc = oc_order[grp * G + l];
+    if (oc >= 0) cnt += (filter[((size_t)oc * C + c0) * kk + p] != 0.f) ? 1 : 0;
   }
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off);
   if (lane == 0) {
-    seg_nnz[seg] = cnt;
-    seg_pad[seg] = (cnt + kBatch - 1) / kBatch * kBatch;
+    grp_nnz[sid] = cnt;
+    grp_pad[sid] = (cnt + kBatch - 1) / kBatch * kBatch;
   }
 }
 
-// exclusive scan of seg_pad into seg_off[0..n], single workgroup
-__global__ __launch_bounds__(1024) void scan_kernel(const int32_t* __restrict__ seg_pad, int32_t* __restrict__ seg_off,
+// exclusive scan of grp_pad into grp_off[0..n], single workgroup
+__global__ __launch_bounds__(1024) void scan_kernel(const int32_t* __restrict__ grp_pad, int32_t* __restrict__ grp_off,
                                                     int n) {
   __shared__ int part[1024];
   const int tid = threadIdx.x;
   const int chunk = (n + 1023) / 1024;
-  const int b = tid * chunk, e = min(n, b + chunk);
+  const int b = min(n, tid * chunk), e = min(n, b + chunk);
   int s = 0;
-  for (int i = b; i < e; ++i) s += seg_pad[i];
+  for (int i = b; i < e; ++i) s += grp_pad[i];
   part[tid] = s;
   __syncthreads();
   for (int off = 1; off < 1024; off <<= 1) {
@@ -55,43 +58,44 @@ __global__ __launch_bounds__(1024) void scan_kernel(const int32_t* __restrict__ 
   }
   int run = tid ? part[tid - 1] : 0;
   for (int i = b; i < e; ++i) {
-    seg_off[i] = run;
-    run += seg_pad[i];
+    grp_off[i] = run;
+    run += grp_pad[i];
   }
-  if (tid == 1023) seg_off[n] = part[1023];
+  if (tid == 1023) grp_off[n] = part[1023];
 }
 
 __global__ __launch_bounds__(256) void scatter_kernel(const float* __restrict__ filter,
                                                       const int32_t* __restrict__ oc_order,
-                                                      const int32_t* __restrict__ seg_off, int32_t* __restrict__ position,
+                                                      const int32_t* __restrict__ grp_off, int32_t* __restrict__ position,
                                                       float* __restrict__ values, int C, int ks, int tile_ic, int stages,
-                                                      int nseg) {
-  const int seg = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+                                                      int G, int nstream) {
+  const int sid = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  if (seg >= nseg) return;
-  const int slot = seg / stages, st = seg - slot * stages;
-  const int oc = oc_order[slot];
-  const int beg = seg_off[seg], end = seg_off[seg + 1];
+  if (sid >= nstream) return;
+  const int grp = sid / stages, st = sid - grp * stages;
+  const int beg = grp_off[sid], end = grp_off[sid + 1];
+  const int kk = ks * ks;
+  const int c0 = st * tile_ic;
+  const int n = min(tile_ic, C - c0) * kk * G;
   int written = 0;
-  if (oc >= 0) {
-    const int kk = ks * ks;
-    const int c0 = st * tile_ic;
-    const int n = min(tile_ic, C - c0) * kk;
-    const float* src = filter + ((size_t)oc * C + c0) * kk;
-    for (int i0 = 0; i0 < n; i0 += 64) {
-      const int i = i0 + lane;
-      const float v = i < n ? src[i] : 0.f;
-      const bool nz = v != 0.f;
-      const unsigned long long m = __ballot(nz);
-      if (nz) {
-        const int rank = __popcll(m & ((1ull << lane) - 1ull));
-        const int ic = i / kk, rs = i - ic * kk;
-        const int r = rs / ks, s = rs - r * ks;
-        position[beg + written + rank] = s + (r << 3) + (ic << 6);
-        values[beg + written + rank] = v;
-      }
-      written += __popcll(m);
+  for (int i0 = 0; i0 < n; i0 += 64) {
+    const int i = i0 + lane;
+    const int p = i / G, l = i - p * G;
+    float v = 0.f;
+    if (i < n) {
+      const int oc = oc_order[grp * G + l];
+      if (oc >= 0) v = filter[((size_t)oc * C + c0) * kk + p];
     }
+    const bool nz = v != 0.f;
+    const unsigned long long m = __ballot(nz);
+    if (nz) {
+      const int rank = __popcll(m & ((1ull << lane) - 1ull));
+      const int ic = p / kk, rs = p - ic * kk;
+      const int r = rs / ks, s = rs - r * ks;
+      position[beg + written + rank] = s + (r << 3) + (ic << 6) + (l << 24);
+      values[beg + written + rank] = v;
+    }
+    written += __popcll(m);
   }
   for (int i = beg + written + lane; i < end; i += 64) {  // padding entries
     position[i] = 0;
@@ -99,29 +103,36 @@ __global__ __launch_bounds__(256) void scatter_kernel(const float* __restrict__ 
   }
 }
 
+// position word -> the kernel's entry code for one tile geometry
 __global__ __launch_bounds__(256) void bind_kernel(const int32_t* __restrict__ position, const float* __restrict__ values,
                                                    int2* __restrict__ out, long long n, int plane, int pitch, int par,
-                                                   int stride) {
+                                                   int stride, int nq) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const int pos = position[i];
-  const int s = pos & 7, r = (pos >> 3) & 7, ic = pos >> 6;
+  const int s = pos & 7, r = (pos >> 3) & 7, ic = (pos >> 6) & 0x3ffff, l = (pos >> 24) & 0xff;
   int2 e;
-  e.x = 4 * (ic * plane + r * pitch + (s % stride) * par + (s / stride) * 4);
+  // [15:0] LDS byte offset, [23:16] first accumulator of the slot, [31:28] VGPR-index enables (see gen_walk_asm.py)
+  e.x = 4 * (ic * plane + r * pitch + (s % stride) * par + (s / stride) * 4) | ((l * 4 * nq) << 16) | (int)0xC0000000u;
   e.y = __float_as_int(values[i]);
   out[i] = e;
 }
 
-int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, const int32_t* oc_order, hipStream_t stream,
-                tetris_g950** out) {
+int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, int G, const int32_t* oc_order,
+                hipStream_t stream, tetris_g950** out) {
   if (!d_filter || !out) return fail(TETRIS_EINVAL, "null argument");
   if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || tile_ic <= 0)
     return fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d tile_ic=%d (ks <= %d)", C, K, ks, tile_ic, kMaxKs);
+  if (G != 4 && G != 8 && G != 16 && G != 32)
+    return fail(TETRIS_EINVAL, "oc_per_wave must be 4, 8, 16 or 32 (got %d)", G);
+  if ((long long)tile_ic * 64 >= (1 << 24))
+    return fail(TETRIS_EINVAL, "tile_ic %d does not fit the position word", tile_ic);
   tetris_g950* p = new tetris_g950;
-  p->C = C; p->K = K; p->ks = ks; p->tile_ic = tile_ic;
+  p->C = C; p->K = K; p->ks = ks; p->tile_ic = tile_ic; p->g = G;
   p->stages = (C - 1) / tile_ic + 1;
-  p->slots = (K + 127) / 128 * 128;
-  const int nseg = p->slots * p->stages;
+  p->slots = (K + kSlotPad - 1) / kSlotPad * kSlotPad;
+  p->groups = p->slots / G;
+  const int nseg = p->groups * p->stages;
 
   std::vector<int32_t> order(p->slots, -1);
   std::vector<char> seen(K, 0);
@@ -147,17 +158,17 @@ int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, const 
       return cleanup(fail(TETRIS_EHIP, "%s failed at %s:%d: %s", #call, __FILE__, __LINE__, hipGetErrorString(e_))); \
   } while (0)
   HIPC(hipMalloc(&p->d_oc_order, sizeof(int32_t) * p->slots));
-  HIPC(hipMalloc(&p->d_seg_off, sizeof(int32_t) * (nseg + 1)));
-  HIPC(hipMalloc(&p->d_seg_nnz, sizeof(int32_t) * nseg));
+  HIPC(hipMalloc(&p->d_grp_off, sizeof(int32_t) * (nseg + 1)));
+  HIPC(hipMalloc(&p->d_grp_nnz, sizeof(int32_t) * nseg));
   HIPC(hipMalloc(&d_pad, sizeof(int32_t) * nseg));
   HIPC(hipMemcpyAsync(p->d_oc_order, order.data(), sizeof(int32_t) * p->slots, hipMemcpyHostToDevice, stream));
   const int blocks = (nseg + 3) / 4;
-  hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, stream, d_filter, p->d_oc_order, p->d_seg_nnz, d_pad, C,
-                     ks, tile_ic, p->stages, nseg);
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, d_pad, p->d_seg_off, nseg);
+  hipLaunchKernelGGL(count_kernel, dim3(blocks), dim3(256), 0, stream, d_filter, p->d_oc_order, p->d_grp_nnz, d_pad, C,
+                     ks, tile_ic, p->stages, G, nseg);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, d_pad, p->d_grp_off, nseg);
   HIPC(hipGetLastError());
   int32_t total = 0;
-  HIPC(hipMemcpyAsync(&total, p->d_seg_off + nseg, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+  HIPC(hipMemcpyAsync(&total, p->d_grp_off + nseg, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
   HIPC(hipStreamSynchronize(stream));
   p->n_entries = total;
   // one spare batch so that a kernel may prefetch the batch after the last one
@@ -165,12 +176,12 @@ int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, const 
   HIPC(hipMalloc(&p->d_values, sizeof(float) * (size_t)(total + kBatch)));
   HIPC(hipMemsetAsync(p->d_position + total, 0, sizeof(int32_t) * kBatch, stream));
   HIPC(hipMemsetAsync(p->d_values + total, 0, sizeof(float) * kBatch, stream));
-  hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(256), 0, stream, d_filter, p->d_oc_order, p->d_seg_off,
-                     p->d_position, p->d_values, C, ks, tile_ic, p->stages, nseg);
+  hipLaunchKernelGGL(scatter_kernel, dim3(blocks), dim3(256), 0, stream, d_filter, p->d_oc_order, p->d_grp_off,
+                     p->d_position, p->d_values, C, ks, tile_ic, p->stages, G, nseg);
   HIPC(hipGetLastError());
   // nnz = sum of seg_nnz, summed on the host (small)
   std::vector<int32_t> nz(nseg);
-  HIPC(hipMemcpyAsync(nz.data(), p->d_seg_nnz, sizeof(int32_t) * nseg, hipMemcpyDeviceToHost, stream));
+  HIPC(hipMemcpyAsync(nz.data(), p->d_grp_nnz, sizeof(int32_t) * nseg, hipMemcpyDeviceToHost, stream));
   HIPC(hipStreamSynchronize(stream));
   p->nnz = 0;
   for (int v : nz) p->nnz += v;
@@ -182,7 +193,7 @@ int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, const 
 }  // namespace
 
 int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** entries_out) {
-  const BoundKey key{g.plane, g.pitch, g.par, g.stride};
+  const BoundKey key{g.plane, g.pitch, g.par, g.stride, g.nq};
   std::lock_guard<std::mutex> lock(p->mu);
   auto it = p->bound.find(key);
   if (it == p->bound.end()) {
@@ -190,7 +201,7 @@ int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** en
     const long long n = p->n_entries + kBatch;
     TETRIS_HIP(hipMalloc(&d, sizeof(int2) * (size_t)n));
     hipLaunchKernelGGL(bind_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p->d_position, p->d_values,
-                       d, n, g.plane, g.pitch, g.par, g.stride);
+                       d, n, g.plane, g.pitch, g.par, g.stride, g.nq);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       (void)hipFree(d);
@@ -206,13 +217,13 @@ int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** en
 
 extern "C" {
 
-int tetris_g950_create_device(const float* d_filter, int C, int K, int ks, int tile_ic, const int32_t* oc_order,
-                              void* stream, tetris_g950** out) {
-  return tetris::pack_device(d_filter, C, K, ks, tile_ic, oc_order, static_cast<hipStream_t>(stream), out);
+int tetris_g950_create_device(const float* d_filter, int C, int K, int ks, int tile_ic, int oc_per_wave,
+                              const int32_t* oc_order, void* stream, tetris_g950** out) {
+  return tetris::pack_device(d_filter, C, K, ks, tile_ic, oc_per_wave, oc_order, static_cast<hipStream_t>(stream), out);
 }
 
-int tetris_g950_create(const float* h_filter, int C, int K, int ks, int tile_ic, const int32_t* oc_order, void* stream,
-                       tetris_g950** out) {
+int tetris_g950_create(const float* h_filter, int C, int K, int ks, int tile_ic, int oc_per_wave,
+                       const int32_t* oc_order, void* stream, tetris_g950** out) {
   if (!h_filter) return tetris::fail(TETRIS_EINVAL, "null filter");
   if (C <= 0 || K <= 0 || ks <= 0) return tetris::fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d", C, K, ks);
   float* d = nullptr;
@@ -220,7 +231,8 @@ int tetris_g950_create(const float* h_filter, int C, int K, int ks, int tile_ic,
   TETRIS_HIP(hipMalloc(&d, bytes));
   hipError_t e = hipMemcpyAsync(d, h_filter, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream));
   int rc = e == hipSuccess ? TETRIS_OK : tetris::fail(TETRIS_EHIP, "filter upload failed: %s", hipGetErrorString(e));
-  if (rc == TETRIS_OK) rc = tetris::pack_device(d, C, K, ks, tile_ic, oc_order, static_cast<hipStream_t>(stream), out);
+  if (rc == TETRIS_OK)
+    rc = tetris::pack_device(d, C, K, ks, tile_ic, oc_per_wave, oc_order, static_cast<hipStream_t>(stream), out);
   (void)hipStreamSynchronize(static_cast<hipStream_t>(stream));
   (void)hipFree(d);
   return rc;
@@ -229,8 +241,8 @@ int tetris_g950_create(const float* h_filter, int C, int K, int ks, int tile_ic,
 void tetris_g950_destroy(tetris_g950* p) {
   if (!p) return;
   for (auto& kv : p->bound) (void)hipFree(kv.second);
-  (void)hipFree(p->d_seg_off);
-  (void)hipFree(p->d_seg_nnz);
+  (void)hipFree(p->d_grp_off);
+  (void)hipFree(p->d_grp_nnz);
   (void)hipFree(p->d_position);
   (void)hipFree(p->d_values);
   (void)hipFree(p->d_oc_order);
@@ -239,28 +251,28 @@ void tetris_g950_destroy(tetris_g950* p) {
 
 int tetris_g950_host_arrays(tetris_g950* p, tetris_g950_arrays* out) {
   if (!p || !out) return tetris::fail(TETRIS_EINVAL, "null argument");
-  const int nseg = p->slots * p->stages;
+  const int nseg = p->groups * p->stages;
   std::lock_guard<std::mutex> lock(p->mu);
-  if (p->h_seg_off.empty()) {
-    p->h_seg_off.resize(nseg + 1);
-    p->h_seg_nnz.resize(nseg);
+  if (p->h_grp_off.empty()) {
+    p->h_grp_off.resize(nseg + 1);
+    p->h_grp_nnz.resize(nseg);
     p->h_position.resize(p->n_entries);
     p->h_values.resize(p->n_entries);
     p->h_oc_order.resize(p->slots);
-    TETRIS_HIP(hipMemcpy(p->h_seg_off.data(), p->d_seg_off, sizeof(int32_t) * (nseg + 1), hipMemcpyDeviceToHost));
-    TETRIS_HIP(hipMemcpy(p->h_seg_nnz.data(), p->d_seg_nnz, sizeof(int32_t) * nseg, hipMemcpyDeviceToHost));
+    TETRIS_HIP(hipMemcpy(p->h_grp_off.data(), p->d_grp_off, sizeof(int32_t) * (nseg + 1), hipMemcpyDeviceToHost));
+    TETRIS_HIP(hipMemcpy(p->h_grp_nnz.data(), p->d_grp_nnz, sizeof(int32_t) * nseg, hipMemcpyDeviceToHost));
     if (p->n_entries) {
       TETRIS_HIP(hipMemcpy(p->h_position.data(), p->d_position, sizeof(int32_t) * p->n_entries, hipMemcpyDeviceToHost));
       TETRIS_HIP(hipMemcpy(p->h_values.data(), p->d_values, sizeof(float) * p->n_entries, hipMemcpyDeviceToHost));
     }
     TETRIS_HIP(hipMemcpy(p->h_oc_order.data(), p->d_oc_order, sizeof(int32_t) * p->slots, hipMemcpyDeviceToHost));
   }
-  out->seg_offsets = p->h_seg_off.data(); out->n_seg_offsets = nseg + 1;
-  out->seg_nnz = p->h_seg_nnz.data();     out->n_seg_nnz = nseg;
+  out->grp_offsets = p->h_grp_off.data(); out->n_grp_offsets = nseg + 1;
+  out->grp_nnz = p->h_grp_nnz.data();     out->n_grp_nnz = nseg;
   out->position = p->h_position.data();   out->n_entries = p->n_entries;
   out->values = p->h_values.data();
   out->oc_order = p->h_oc_order.data();   out->n_slots = p->slots;
-  out->stages = p->stages; out->tile_ic = p->tile_ic; out->nnz = p->nnz;
+  out->stages = p->stages; out->tile_ic = p->tile_ic; out->oc_per_wave = p->g; out->nnz = p->nnz;
   return TETRIS_OK;
 }
 

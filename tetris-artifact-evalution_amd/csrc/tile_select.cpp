@@ -5,6 +5,8 @@
 // TILE_W} instantiations (Tetris/spconv2d.cc:90-329, 130 launches and one re-pack per candidate).
 #include <algorithm>
 #include <climits>
+#include <cmath>
+#include <utility>
 
 #include "common.h"
 
@@ -12,23 +14,55 @@ namespace tetris {
 
 namespace {
 
-constexpr int kLdsLimit = 160 * 1024;
+struct Shape {
+  int lw, lr, lh, thi, nb, ng, par, pitch, ih;
+};
 
-// LDS serves a 16-byte-per-lane read in groups of lanes over 64 four-byte banks.  Score a row pitch by
-// the worst bank multiplicity inside each group of 16 consecutive lanes (1 = conflict free).
-int bank_cost(int lw, int lh, int stride, int pitch) {
-  int cost = 0;
-  for (int g0 = 0; g0 < 64; g0 += 16) {
-    int banks[64] = {0};
-    for (int l = g0; l < g0 + 16; ++l) {
-      const int lx = l % lw, ly = l / lw;
-      if (ly >= lh) continue;
-      const int dw = ly * stride * pitch + lx * 4;
-      for (int j = 0; j < 4; ++j) banks[(dw + j) & 63] += 1;
+// Period (in dwords) of the bank rule for `lr` lane positions per row: 64, except that rows of 1, 2 or 4
+// lanes repeat every 8 * lr dwords (measured with 16-byte reads on MI355X).
+inline int bank_period(int lr) { return (lr == 1 || lr == 2 || lr == 4) ? 8 * lr : 64; }
+
+// Lane rows and LDS pitch for `lw` active lanes per row.  The LDS distance between consecutive lane rows,
+// stride * pitch dwords, must equal 4 * lr modulo the bank period for full-rate 16-byte reads; among the
+// (lr, pitch) pairs that satisfy it, take the one that wastes the least: idle lane positions cost compute
+// time one for one, a padded pitch only costs LDS room.
+Shape unit_shape(int lw, int OH, int N, int ks, int stride) {
+  Shape s;
+  s.lw = lw;
+  s.ng = lw + (ks - 1) / stride;
+  s.par = 4 * s.ng;
+  const int min_pitch = stride * s.par;
+  double best = 1e300;
+  s.lr = lw;
+  s.pitch = min_pitch;
+  for (int lr = lw; lr <= 64 && lr <= lw + 16; ++lr)
+    for (int pitch = min_pitch; pitch <= min_pitch + 64; pitch += 4) {
+      if ((stride * pitch - 4 * lr) % bank_period(lr) != 0) continue;
+      const int lh = 64 / lr;
+      const int thi = std::min(lh, OH);
+      const int rows = std::max(1, std::min(lh / thi, N)) * thi;  // lane rows that can hold pixels
+      const double cost = (64.0 / (rows * lw)) * (1.0 + 0.25 * ((double)pitch / min_pitch - 1.0));
+      if (cost < best - 1e-9) {
+        best = cost;
+        s.lr = lr;
+        s.pitch = pitch;
+      }
+      break;  // larger pitches with this lr only cost more
     }
-    cost += *std::max_element(banks, banks + 64);
-  }
-  return cost;
+  s.lh = 64 / s.lr;
+  s.thi = std::min(s.lh, OH);
+  s.nb = std::max(1, std::min(s.lh / s.thi, N));
+  s.ih = stride * (s.thi - 1) + ks;
+  return s;
+}
+
+// Dwords per image of a unit's region: at least tile_ic planes, padded so that the step from the last lane
+// row of one image to the first of the next also meets the bank rule.
+int image_stride(const Shape& s, int tile_ic, int stride) {
+  int v = tile_ic * s.ih * s.pitch;
+  if (s.nb > 1)
+    while ((v - (s.thi - 1) * stride * s.pitch - 4 * s.lr) % bank_period(s.lr) != 0) v += 4;
+  return v;
 }
 
 }  // namespace
@@ -42,91 +76,147 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   g.OW = out_extent(W, pad, p->ks, stride);
   if (H + 2 * pad < p->ks || W + 2 * pad < p->ks || g.OH <= 0 || g.OW <= 0)
     return fail(TETRIS_EINVAL, "kernel %d does not fit the padded %dx%d image", p->ks, H, W);
-  if ((long long)N * p->C * H * W >= INT_MAX || (long long)N * p->K * g.OH * g.OW >= (1ll << 40))
-    return fail(TETRIS_EINVAL, "tensor too large for 32-bit in-tile offsets");
   g.tile_ic = p->tile_ic;
   g.stages = p->stages;
   g.slots = p->slots;
 
-  const int nq = t.quads;
-  if (t.lanes_w < 1 || t.lanes_w > 64 || (nq != 1 && nq != 2 && nq != 4))
-    return fail(TETRIS_EINVAL, "bad tile: lanes_w=%d quads=%d", t.lanes_w, nq);
-  if ((t.oc_per_wave != 4 && t.oc_per_wave != 8 && t.oc_per_wave != 16) ||
-      (t.waves != 1 && t.waves != 2 && t.waves != 4 && t.waves != 8))
-    return fail(TETRIS_EINVAL, "bad tile: oc_per_wave=%d waves=%d", t.oc_per_wave, t.waves);
-  g.lw = t.lanes_w;
-  g.lh = 64 / g.lw;
-  const int vrows = nq * g.lh;
-  g.thi = std::min(vrows, g.OH);
-  g.nb = std::max(1, std::min(vrows / g.thi, N));
-  g.ng = g.lw + (p->ks - 1) / stride;
-  g.par = 4 * g.ng;
-  const int min_pitch = stride * g.par;
-  int best_pitch = min_pitch, best_cost = INT_MAX;
-  for (int pitch = min_pitch; pitch <= min_pitch + min_pitch / 4 + 4; pitch += 4) {
-    const int c = bank_cost(g.lw, g.lh, stride, pitch);
-    if (c < best_cost) {
-      best_cost = c;
-      best_pitch = pitch;
-    }
-  }
-  g.pitch = best_pitch;
-  g.ih = stride * (g.thi - 1) + p->ks;
+  g.nq = t.quads;
+  g.g = p->g;
+  g.waves = t.waves;
+  if (t.lanes_w < 1 || t.lanes_w > 64 || (g.nq != 1 && g.nq != 2 && g.nq != 4))
+    return fail(TETRIS_EINVAL, "bad tile: lanes_w=%d quads=%d", t.lanes_w, g.nq);
+  if (t.oc_per_wave != p->g)
+    return fail(TETRIS_EINVAL, "tile wants %d output channels per wave, the pack was made for %d", t.oc_per_wave, p->g);
+  if (g.g * 4 * g.nq > kAccRegs)
+    return fail(TETRIS_EINVAL, "oc_per_wave * 4 * quads = %d exceeds the %d accumulators of a wave", g.g * 4 * g.nq,
+                kAccRegs);
+  if (t.waves != 1 && t.waves != 2 && t.waves != 4 && t.waves != 8)
+    return fail(TETRIS_EINVAL, "bad tile: waves=%d (1, 2, 4 or 8)", t.waves);
+  const Shape s = unit_shape(t.lanes_w, g.OH, N, p->ks, stride);
+  g.lw = s.lw; g.lr = s.lr; g.lh = s.lh; g.thi = s.thi; g.nb = s.nb; g.ng = s.ng; g.par = s.par; g.ih = s.ih;
+  g.region = kTileBytes / g.nq;
+  g.pitch = s.pitch;
   g.plane = g.ih * g.pitch;
-  g.img_stride = g.tile_ic * g.plane;
-  g.fill_slots = g.nb * g.ih * stride * g.ng;
-  g.tiles_w = ceil_div(g.OW, 4 * g.lw);
-  g.tiles_h = ceil_div(g.OH, g.thi);
-  g.tiles_n = ceil_div(N, g.nb);
-  g.kb = t.waves * t.oc_per_wave;
+  g.img_stride = image_stride(s, g.tile_ic, stride);
+  if (4ll * g.nb * g.img_stride > g.region)
+    return fail(TETRIS_EINVAL, "a pixel unit needs %lld bytes of LDS for %d staged channels (region is %d): lower tile_ic "
+                "or quads", 4ll * g.nb * g.img_stride, g.tile_ic, g.region);
+  g.units_w = ceil_div(g.OW, 4 * g.lw);
+  g.units_h = ceil_div(g.OH, g.thi);
+  g.units_n = ceil_div(N, g.nb);
+  const long long units = (long long)g.units_w * g.units_h * g.units_n;
+  g.kb = t.waves * g.g;
   g.kblocks = ceil_div(p->K, g.kb);
   if (g.kblocks * g.kb > p->slots) return fail(TETRIS_EINVAL, "channel block %d does not divide the slot padding", g.kb);
-  const long long lds = 4ll * g.nb * g.img_stride + 20ll * g.fill_slots;
-  if (lds > kLdsLimit)
-    return fail(TETRIS_EINVAL, "tile needs %lld bytes of LDS (limit %d): lower tile_ic, quads or lanes_w", lds,
-                kLdsLimit);
-  g.lds_bytes = (int)lds;
-  if ((long long)g.tiles_n * g.tiles_h * g.tiles_w * g.kblocks > (1ll << 30))
-    return fail(TETRIS_EINVAL, "grid too large");
+  if (units * g.kblocks > (1ll << 30)) return fail(TETRIS_EINVAL, "grid too large");
+  g.units = (int)units;
+  g.ugroups = ceil_div(g.units, g.nq);
+  // a workgroup addresses its images through one 2 GB buffer window
+  const long long img_bytes = 4ll * p->C * H * W;
+  if (img_bytes * ((long long)g.nq * g.nb + 2) >= (1ll << 31))
+    return fail(TETRIS_EINVAL, "images too large for the 2 GB input window of a workgroup");
+  if ((long long)N * p->K * g.OH * g.OW >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
+  // staging plan
+  g.slots_per_unit = g.nb * g.ih * stride * g.ng;
+  g.fill_slots = g.nq * g.slots_per_unit;
+  const int threads = t.waves * 64;
+  if (g.fill_slots <= threads) {
+    g.spt = 1;
+    g.cg = std::min(threads / g.fill_slots, g.tile_ic);
+  } else {
+    g.spt = 2;
+    g.cg = 1;
+    if (g.fill_slots > 2 * threads)
+      return fail(TETRIS_EINVAL, "%d LDS slots per stage are more than %d threads can stage: use more waves or fewer "
+                  "quads", g.fill_slots, threads);
+  }
+  g.fill_iters = ceil_div(g.tile_ic, g.cg);
+  if (g.spt * g.fill_iters > kFillItems)
+    return fail(TETRIS_EINVAL, "staging %d channels takes %d loads per thread (limit %d): lower tile_ic or use more "
+                "waves", g.tile_ic, g.spt * g.fill_iters, kFillItems);
   *out = g;
   return TETRIS_OK;
 }
 
-int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t) {
+// Largest tile_ic (a power of two, or C itself when smaller) that a tile shape can stage.
+static int max_tile_ic(const Shape& s, int nq, int waves, int stride, int C) {
+  const int region = kTileBytes / nq;
+  const int threads = waves * 64;
+  const int fill_slots = nq * s.nb * s.ih * stride * s.ng;
+  if (fill_slots > 2 * threads) return 0;
+  int best = 0;
+  for (int t = 1; t <= 256; t *= 2) {
+    const int tic = std::min(t, C);
+    if (4ll * s.nb * image_stride(s, tic, stride) > region) break;
+    int spt, cg;
+    if (fill_slots <= threads) { spt = 1; cg = std::min(threads / fill_slots, tic); } else { spt = 2; cg = 1; }
+    if (spt * ceil_div(tic, cg) > kFillItems) break;
+    best = tic;
+    if (tic == C) break;
+  }
+  return best;
+}
+
+int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad layer shape");
   const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
   if (OH <= 0 || OW <= 0) return fail(TETRIS_EINVAL, "empty output");
-  tetris_tile best{};
-  best.quads = 2;
-  best.oc_per_wave = 8;
-  best.waves = 4;
-  while (best.waves > 1 && best.waves * best.oc_per_wave / 2 >= K) best.waves /= 2;
-  // lanes across: least padded pixel slots, then the widest rows
-  long long best_slots = LLONG_MAX;
-  const int cand[] = {16, 14, 13, 8, 7, 4, 2, 1};
-  for (int lw : cand) {
-    const int lh = 64 / lw, vrows = best.quads * lh;
-    const int thi = std::min(vrows, OH);
-    const int nb = std::max(1, std::min(vrows / thi, N));
-    const long long tiles = (long long)ceil_div(OW, 4 * lw) * ceil_div(OH, thi) * ceil_div(N, nb);
-    const long long slots = tiles * 64 * best.quads * 4;
-    if (slots < best_slots) {
-      best_slots = slots;
-      best.lanes_w = lw;
+  // Score every candidate with a small time model calibrated on MI355X and keep the cheapest:
+  //   a wave spends about 35 + 41 * quads cycles per entry when two waves share a SIMD (one LDS dword per
+  //   FMA is what binds it) and about 0.62 of that when it has the SIMD to itself; a stage costs about 2000
+  //   cycles of barriers and stream start-up plus 60 per 16-byte slot a thread stages, and the waves of a
+  //   workgroup wait for the slowest one at every stage; a CU holds eight waves.
+  static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}};
+  static const int kWaves[] = {8, 4, 2, 1};
+  const double density = 0.15;  // the mask is not known here; typical of the pruned layers this runs
+  std::vector<std::pair<double, tetris_tile>> scored;
+  for (int lw = 1; lw <= 62; ++lw) {
+    if (4 * (lw - 1) >= OW && lw > 1) break;  // wider than the image
+    if (4 * lw < (OW >= 28 ? 28 : (OW + 1) / 2)) continue;  // narrow tiles stage their halo'd rows poorly (measured)
+    const Shape s = unit_shape(lw, OH, N, ks, stride);
+    const long long units = (long long)ceil_div(OW, 4 * lw) * ceil_div(OH, s.thi) * ceil_div(N, s.nb);
+    for (const auto& qg : kQuadG) {
+      const int nq = qg[0], g = qg[1];
+      for (int waves : kWaves) {
+        const int kb = waves * g;
+        if (kb > kSlotPad) continue;
+        const int tic_max = max_tile_ic(s, nq, waves, stride, C);
+        if (tic_max <= 0) continue;
+        for (int tic = tic_max, tries = 0; tic >= 1 && tries < 3; tic /= 2, ++tries) {  // fewer channels, more stages
+        const long long ugroups = (units + nq - 1) / nq;
+        const int kblocks = ceil_div(K, kb);
+        const int stages = ceil_div(C, tic);
+        const double entries = g * tic * ks * ks * density + 4.0;  // per wave and stage, with stream padding
+        // waves of a workgroup meet at a barrier every stage: the slowest of them sets the pace
+        const double straggle = waves > 1 ? 1.4 * std::sqrt(entries) : 0.0;
+        const double items = (double)tic * nq * s.nb * s.ih * stride * s.ng / (waves * 64);  // staged slots per thread
+        const double per_wave = stages * ((entries + straggle) * (35.0 + 41.0 * nq) + 2000.0 + 60.0 * items);
+        const double waves_total = (double)ugroups * kblocks * waves;
+        const double rounds = waves_total / (256.0 * 8.0);
+        // input re-read by every channel block, in units of the per-wave cycle count (a weak tie-breaker)
+        const double reread = 1.0 + 0.02 * kblocks;
+        const double cost = per_wave * std::max(rounds, 0.62) * reread;
+        tetris_tile t{};
+        t.lanes_w = lw; t.quads = nq; t.oc_per_wave = g; t.waves = waves; t.tile_ic = tic;
+        scored.emplace_back(cost, t);
+        }
+      }
     }
   }
-  // input channels per stage: the most that keeps three workgroups per CU resident
-  const int lw = best.lanes_w, lh = 64 / lw, vrows = best.quads * lh;
-  const int thi = std::min(vrows, OH), nb = std::max(1, std::min(vrows / thi, N));
-  const int ih = stride * (thi - 1) + ks;
-  const int pitch = stride * 4 * (lw + (ks - 1) / stride);
-  const long long per_ic = 4ll * nb * ih * (pitch + pitch / 8);
-  int tile_ic = 64;
-  while (tile_ic > 4 && per_ic * tile_ic > 50 * 1024) tile_ic /= 2;
-  while (tile_ic > 4 && tile_ic / 2 >= C) tile_ic /= 2;
-  best.tile_ic = tile_ic;
-  *t = best;
+  if (scored.empty()) return fail(TETRIS_EINVAL, "no tile shape fits this layer");
+  std::stable_sort(scored.begin(), scored.end(),
+                   [](const std::pair<double, tetris_tile>& a, const std::pair<double, tetris_tile>& b) { return a.first < b.first; });
+  ranked->clear();
+  for (const auto& e : scored) ranked->push_back(e.second);
+  return TETRIS_OK;
+}
+
+int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t) {
+  std::vector<tetris_tile> ranked;
+  const int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked);
+  if (rc) return rc;
+  *t = ranked[0];
   return TETRIS_OK;
 }
 

@@ -62,10 +62,10 @@ class _SpfArrays(C.Structure):
 
 
 class _G950Arrays(C.Structure):
-    _fields_ = [("seg_offsets", C.c_void_p), ("n_seg_offsets", C.c_int64), ("seg_nnz", C.c_void_p),
-                ("n_seg_nnz", C.c_int64), ("position", C.c_void_p), ("n_entries", C.c_int64), ("values", C.c_void_p),
+    _fields_ = [("grp_offsets", C.c_void_p), ("n_grp_offsets", C.c_int64), ("grp_nnz", C.c_void_p),
+                ("n_grp_nnz", C.c_int64), ("position", C.c_void_p), ("n_entries", C.c_int64), ("values", C.c_void_p),
                 ("oc_order", C.c_void_p), ("n_slots", C.c_int64), ("stages", C.c_int32), ("tile_ic", C.c_int32),
-                ("nnz", C.c_int64)]
+                ("oc_per_wave", C.c_int32), ("nnz", C.c_int64)]
 
 
 class Tile(C.Structure):
@@ -89,14 +89,15 @@ _lib.tetris_spf_destroy.argtypes = [C.c_void_p]
 _lib.tetris_spf_destroy.restype = None
 _lib.tetris_spf_host_arrays.argtypes = [C.c_void_p, C.POINTER(_SpfArrays)]
 _lib.tetris_spf_device_arrays.argtypes = [C.c_void_p, C.POINTER(_SpfArrays)]
-_lib.tetris_g950_create.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, _i32p_opt, C.c_void_p,
+_lib.tetris_g950_create.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i32p_opt, C.c_void_p,
                                     C.POINTER(C.c_void_p)]
-_lib.tetris_g950_create_device.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, _i32p_opt, C.c_void_p,
-                                           C.POINTER(C.c_void_p)]
+_lib.tetris_g950_create_device.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i32p_opt,
+                                           C.c_void_p, C.POINTER(C.c_void_p)]
 _lib.tetris_g950_destroy.argtypes = [C.c_void_p]
 _lib.tetris_g950_destroy.restype = None
 _lib.tetris_g950_host_arrays.argtypes = [C.c_void_p, C.POINTER(_G950Arrays)]
 _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
+_lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
 _lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile),
                                                                                                 C.c_void_p]
 _lib.tetris_spconv2d_launch_spf.argtypes = [C.c_void_p] * 7 + [C.c_int] * 8 + [C.c_void_p]
@@ -193,9 +194,15 @@ class SparseFilter:
 
 
 class G950Filter:
-    """The gfx950 pack the HIP kernel consumes (tetris_g950_create / _create_device)."""
+    """The gfx950 pack the HIP kernel consumes (tetris_g950_create / _create_device).
 
-    def __init__(self, filter, tile_ic, oc_order=None, stream=0, device_ptr=None, shape=None):
+    `G950Filter.for_tile(filter, tile)` makes the pack that a Tile from tile_select() needs."""
+
+    @classmethod
+    def for_tile(cls, filter, tile, oc_order=None, stream=0):
+        return cls(filter, tile.tile_ic, tile.oc_per_wave, oc_order, stream)
+
+    def __init__(self, filter, tile_ic, oc_per_wave, oc_order=None, stream=0, device_ptr=None, shape=None):
         if device_ptr is None:
             w = np.ascontiguousarray(filter, np.float32)
             K, Cc, ks, _ = w.shape
@@ -205,21 +212,22 @@ class G950Filter:
         optr = None if order is None else order.ctypes.data_as(C.c_void_p)
         self._h = C.c_void_p()
         if device_ptr is None:
-            _check(_lib.tetris_g950_create(w, Cc, K, ks, tile_ic, optr, C.c_void_p(stream), C.byref(self._h)))
+            _check(_lib.tetris_g950_create(w, Cc, K, ks, tile_ic, oc_per_wave, optr, C.c_void_p(stream),
+                                           C.byref(self._h)))
         else:
-            _check(_lib.tetris_g950_create_device(C.c_void_p(device_ptr), Cc, K, ks, tile_ic, optr, C.c_void_p(stream),
-                                                  C.byref(self._h)))
-        self.K, self.C, self.ks, self.tile_ic = K, Cc, ks, tile_ic
+            _check(_lib.tetris_g950_create_device(C.c_void_p(device_ptr), Cc, K, ks, tile_ic, oc_per_wave, optr,
+                                                  C.c_void_p(stream), C.byref(self._h)))
+        self.K, self.C, self.ks, self.tile_ic, self.oc_per_wave = K, Cc, ks, tile_ic, oc_per_wave
 
     def host_arrays(self):
         a = _G950Arrays()
         _check(_lib.tetris_g950_host_arrays(self._h, C.byref(a)))
-        return dict(seg_offsets=_np_view(a.seg_offsets, a.n_seg_offsets, np.int32),
-                    seg_nnz=_np_view(a.seg_nnz, a.n_seg_nnz, np.int32),
+        return dict(grp_offsets=_np_view(a.grp_offsets, a.n_grp_offsets, np.int32),
+                    grp_nnz=_np_view(a.grp_nnz, a.n_grp_nnz, np.int32),
                     position=_np_view(a.position, a.n_entries, np.int32),
                     values=_np_view(a.values, a.n_entries, np.float32),
                     oc_order=_np_view(a.oc_order, a.n_slots, np.int32), stages=int(a.stages), tile_ic=int(a.tile_ic),
-                    nnz=int(a.nnz))
+                    oc_per_wave=int(a.oc_per_wave), nnz=int(a.nnz))
 
     def launch(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0):
         """Asynchronous conv on raw device pointers (NCHW in, NCHW out)."""
@@ -247,6 +255,16 @@ def tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, strid
     _check(_lib.tetris_tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
                                    C.byref(t)))
     return t
+
+
+def tile_autotune(filter, batch, img_h, img_w, stride, padding, max_candidates=0, stream=0):
+    """-> (Tile, ms per launch) of the fastest measured tile shape for this filter and input shape."""
+    w = np.ascontiguousarray(filter, np.float32)
+    K, Cc, ks, _ = w.shape
+    t, ms = Tile(), C.c_float()
+    _check(_lib.tetris_tile_autotune(w, batch, img_h, img_w, Cc, K, ks, stride, padding, max_candidates,
+                                     C.c_void_p(stream), C.byref(t), C.byref(ms)))
+    return t, float(ms.value)
 
 
 def SparseConv2d(input, offsets, stage_len, oc_permutation, position, values, output, batch_size, img_h, img_w,
