@@ -23,9 +23,9 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 PEAK_HBM_GBS = 8000.0        # MI355X published HBM3E bandwidth
 PEAK_FP32_TFLOPS = 157.3     # MI355X published vector/matrix fp32 peak
 
-# HBM bytes per step (all launches of spconv2d_kernel) from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
+# HBM bytes per launch of spconv2d_kernel (average over a step) from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of this file, scaled by the same counters on a copy kernel of known size; see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.174e8}  # average per launch over the 16 layers
 
 
 def main():
@@ -42,6 +42,12 @@ def main():
                     help="autotune: time the selector's best candidates per layer during set-up (what the reference's "
                          "driver does with its 185-entry table); select: take the selector's first choice unmeasured")
     ap.add_argument("--candidates", type=int, default=24)
+    ap.add_argument("--save-tiles", metavar="FILE", help="write the tile chosen for every layer to FILE (JSON)")
+    ap.add_argument("--load-tiles", metavar="FILE", help="use the tiles a previous --save-tiles run wrote (so that a "
+                    "profiled run launches nothing but packing and the timed convolutions)")
+    ap.add_argument("--calibrate-copy", type=int, metavar="MIB", default=0,
+                    help="instead of the benchmark, run one elementwise copy kernel over MIB MiB (reads MIB, writes MIB): "
+                         "the known-size dispatch that scales the FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this engine runs on one GPU (no collectives or sharding are part of the path); "
@@ -56,14 +62,30 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
+    if args.calibrate_copy:
+        n = args.calibrate_copy * (1 << 20) // 4
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(4):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_mib": args.calibrate_copy, "dispatches": 4,
+                          "bytes_read_per_dispatch": 4 * n, "bytes_written_per_dispatch": 4 * n}))
+        return
     layers = W.SUITES[args.suite]()
     N = args.batch
 
     packs, tiles, xs, ys, works = [], [], [], [], []
     t_pack = 0.0
-    for L in layers:
+    loaded = json.load(open(args.load_tiles)) if args.load_tiles else None
+    if loaded is not None and (loaded["suite"], loaded["batch"], len(loaded["tiles"])) != (args.suite, N, len(layers)):
+        sys.exit("bench.py: %s was written for another workload" % args.load_tiles)
+    for li, L in enumerate(layers):
         w = W.make_weights(L)
-        if args.tile == "autotune":
+        if loaded is not None:
+            tile = T.Tile(*loaded["tiles"][li])
+        elif args.tile == "autotune":
             tile, _ = T.tile_autotune(w, N, L.H, L.W, L.stride, L.pad, args.candidates)
         else:
             tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
@@ -76,6 +98,10 @@ def main():
         y = torch.empty((N, L.K, oh, ow), dtype=torch.float32, device=dev)
         packs.append(pk); tiles.append(tile); xs.append(x); ys.append(y); works.append(W.work(L, N))
     torch.cuda.synchronize()
+    if args.save_tiles:
+        with open(args.save_tiles, "w") as f:
+            json.dump({"suite": args.suite, "batch": N,
+                       "tiles": [[t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic] for t in tiles]}, f)
 
     def step():
         for L, pk, tile, x, y in zip(layers, packs, tiles, xs, ys):
@@ -83,12 +109,17 @@ def main():
 
     for _ in range(args.warmup):
         step()
+    # The launches go to the null stream, which is torch's current stream here, so torch's events bracket them.
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    ev0.record()
     for _ in range(args.steps):
         step()
+    ev1.record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step_dev = ev0.elapsed_time(ev1) / args.steps  # device-side span of the same K steps
 
     # spot check of one mid-sized layer against the CPU oracle (not timed)
     check = None
@@ -107,6 +138,8 @@ def main():
     table = []
     t_layers = 0.0
     for L, pk, tile, x, y, wk in zip(layers, packs, tiles, xs, ys, works):
+        if args.layer_repeat <= 0:
+            break
         ms = pk.time(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile, warm=5, repeat=args.layer_repeat)
         t = ms * 1e-3
         t_layers += t
@@ -120,23 +153,26 @@ def main():
     bytes_alg = sum(w["bytes"] for w in works)
     t_roof = sum(w["t_roof"] for w in works)
     n_launch = len(layers)
+    # Average launch duration of the conv kernel over the timed region: the device-side span of the K steps
+    # (events on the launch stream) divided by the launches in it; nothing else runs on the stream in between.
+    t_step = ms_per_step_dev * 1e-3
     t_hbm, t_fp32 = bytes_alg / (PEAK_HBM_GBS * 1e9), fl_sparse / (PEAK_FP32_TFLOPS * 1e12)
     if t_fp32 >= t_hbm:
-        achieved = fl_sparse / t_layers / 1e12
+        achieved = fl_sparse / t_step / 1e12
         roofline = {"bound": "mfma", "bound_detail": "vector fp32 FMA issued from the VALU; no MFMA is used. Peak is the "
                     "published 157.3 TFLOP/s fp32 figure, which needs packed fp32 FMA; this build compiles with packed "
                     "fp32 off, so 78.6 TFLOP/s is the most its instructions can reach",
                     "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP32_TFLOPS, 4)}
     else:
-        achieved = bytes_alg / t_layers / 1e9
+        achieved = bytes_alg / t_step / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(achieved / PEAK_HBM_GBS, 4)}
     roofline.update({"kernel": "spconv2d_kernel", "launches_per_step": n_launch,
-                     "avg_launch_us": round(t_layers / n_launch * 1e6, 2),
+                     "avg_launch_us": round(t_step / n_launch * 1e6, 2),
                      "algorithmic_flops_per_launch": fl_sparse / n_launch,
                      "algorithmic_bytes_per_launch": bytes_alg / n_launch,
-                     "sum_of_layer_roofs_frac": round(t_roof / t_layers, 4),
+                     "sum_of_layer_roofs_frac": round(t_roof / t_step, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get("%s/%d" % (args.suite, N))})
 
     cpu = None
@@ -175,11 +211,12 @@ def main():
         "value": round(fl_dense / (ms_per_step * 1e-3) / 1e9, 1),
         "unit": "GFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_device": round(ms_per_step_dev, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s-shaped sparse conv stack, %d layers, batch %d, fp32 NCHW, seeded unstructured masks"
                    % (args.suite, len(layers), N), "suite": args.suite, "batch": N, "layers": len(layers)},
         "sparse_gflops": round(fl_sparse / (ms_per_step * 1e-3) / 1e9, 1),
-        "sum_layer_us": round(t_layers * 1e6, 1),
+        "sum_layer_us": round(t_layers * 1e6, 1) if table else None,
         "pack_ms_total": round(t_pack * 1e3, 2),
         "tile_selection": args.tile,
         "roofline": roofline,

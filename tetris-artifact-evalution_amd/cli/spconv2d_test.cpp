@@ -1,0 +1,139 @@
+// spconv2d_test <weight_file> [batch] [--seed S] [--dump FILE]      (built twice: spconv2d_test and, with
+// -DTETRIS_CLI_SPF, spf_test)
+//
+// Counterpart of the reference's per-layer binaries: main of Tetris/spconv2d.cc:369-450 (spconv2d_test.o,
+// "Time of Spconv2d :<ms>ms" / "FLOPS of Spconv2d :<x>T") and of Tetris/spf.cc:95-176 (spf_test.o,
+// "Time of Ablation :<ms>ms").  It reads one pruned layer in the reference's text format, makes a random
+// input, runs the host-to-host entry point (upload, pack, tile selection, 30 warm-up + 100 timed
+// launches, download) and prints the same lines, so a loop over weight files that parses the reference's
+// stdout (evalution/conv2d_timing.py:51-79) can drive it unchanged.
+//
+// The reference seeds rand() with time(0) (Tetris/spconv2d.cc:377); here the input comes from a
+// seeded generator so that a run can be repeated, and --dump writes input and output tensors (raw
+// fp32: N*C*H*W inputs, then N*K*OH*OW outputs, both NCHW) for an external checker.  Like the
+// reference's shipped builds (BENCHMARK is defined in Tetris/tensor_utils.h:8) no CPU convolution is
+// run here.
+#include <hip/hip_runtime_api.h>
+
+#include <cassert>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <iostream>
+#include <string>
+
+#define BANK_OPTIMIZE        // the production variant: evalution/script/build_all.sh:14
+#define REORDER_OUT_CHANNEL
+#include "tetris_spconv2d.hpp"
+
+namespace {
+
+struct SplitMix64 {
+  uint64_t s;
+  uint64_t next() {
+    uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+  }
+};
+
+// uniform in [-1, 1), the range of the reference's RandFloat (Tetris/tensor_utils.cc:9-14)
+void GenRandTensor(float* t, size_t len, uint64_t seed) {
+  SplitMix64 g{seed};
+  for (size_t i = 0; i < len; ++i) t[i] = static_cast<float>(g.next() >> 40) * (2.0f / 16777216.0f) - 1.0f;
+}
+
+#define CLI_HIP(call)                                                                              \
+  do {                                                                                             \
+    hipError_t e_ = (call);                                                                        \
+    if (e_ != hipSuccess) {                                                                        \
+      std::fprintf(stderr, "HIP error at %s %d: %s\n", __FILE__, __LINE__, hipGetErrorString(e_)); \
+      std::exit(EXIT_FAILURE);                                                                     \
+    }                                                                                              \
+  } while (0)
+
+}  // namespace
+
+int main(int argc, char* argv[]) {
+  std::cout << "args : " << argc;
+  for (int i = 0; i < argc; ++i) std::cout << " " << argv[i];
+  std::cout << "\n\n";
+
+  std::string weight_file, dump;
+  int batch_size = 4;
+  uint64_t seed = 1;
+  int positional = 0;
+  for (int i = 1; i < argc; ++i) {
+    if (!std::strcmp(argv[i], "--seed") && i + 1 < argc) {
+      seed = std::strtoull(argv[++i], nullptr, 10);
+    } else if (!std::strcmp(argv[i], "--dump") && i + 1 < argc) {
+      dump = argv[++i];
+    } else if (positional == 0) {
+      weight_file = argv[i];
+      ++positional;
+    } else if (positional == 1) {
+      batch_size = std::atoi(argv[i]);
+      ++positional;
+    } else {
+      std::fprintf(stderr, "usage: %s <weight_file> [batch] [--seed S] [--dump FILE]\n", argv[0]);
+      return 2;
+    }
+  }
+  if (weight_file.empty() || batch_size <= 0) {
+    std::fprintf(stderr, "usage: %s <weight_file> [batch] [--seed S] [--dump FILE]\n", argv[0]);
+    return 2;
+  }
+
+  const int dev_id = 0;
+  hipDeviceProp_t prop;
+  CLI_HIP(hipSetDevice(dev_id));
+  CLI_HIP(hipGetDeviceProperties(&prop, dev_id));
+  std::printf("GPU Device %d: \"%s\" (%s, %d compute units)\n\n", dev_id, prop.name, prop.gcnArchName,
+              prop.multiProcessorCount);
+  std::fflush(stdout);
+
+  const std::string layout = "NHWC";  // what the reference's mains pass; host tensors stay NCHW
+  const bool apply_reorder = true;
+  int in_channel, img_h, img_w, kernel_size, out_channel, stride, padding, groups;
+  float* h_filter = ReadConfigAndDataFromFile(weight_file, batch_size, layout, img_h, img_w, in_channel, out_channel,
+                                              kernel_size, stride, padding, groups);
+
+  const int out_h = (img_h + padding * 2 - kernel_size) / stride + 1;
+  const int out_w = (img_w + padding * 2 - kernel_size) / stride + 1;
+  const size_t n_in = (size_t)batch_size * in_channel * img_h * img_w;
+  const size_t n_out = (size_t)batch_size * out_h * out_w * out_channel;
+  float* h_input = static_cast<float*>(std::malloc(n_in * sizeof(float)));
+  float* h_sparse = static_cast<float*>(std::malloc(n_out * sizeof(float)));
+  if (!h_input || !h_sparse) {
+    std::fprintf(stderr, "out of host memory\n");
+    return 1;
+  }
+  GenRandTensor(h_input, n_in, seed);
+
+  hipStream_t stream;
+  CLI_HIP(hipStreamCreate(&stream));
+#ifdef TETRIS_CLI_SPF
+  SparseConv2d_SPF<float, int, int>(h_input, h_filter, h_sparse, batch_size, img_h, img_w, in_channel, out_channel,
+                                    kernel_size, stride, padding, stream, layout, apply_reorder);
+#else
+  CudaSparseConv2d<float, int, int>(h_input, h_filter, h_sparse, batch_size, img_h, img_w, in_channel, out_channel,
+                                    kernel_size, stride, padding, stream, layout, apply_reorder);
+#endif
+  CLI_HIP(hipStreamDestroy(stream));
+
+  if (!dump.empty()) {
+    FILE* fp = std::fopen(dump.c_str(), "wb");
+    if (!fp || std::fwrite(h_input, sizeof(float), n_in, fp) != n_in ||
+        std::fwrite(h_sparse, sizeof(float), n_out, fp) != n_out) {
+      std::fprintf(stderr, "cannot write %s\n", dump.c_str());
+      return 1;
+    }
+    std::fclose(fp);
+  }
+  std::free(h_input);
+  std::free(h_filter);
+  std::free(h_sparse);
+  return 0;
+}

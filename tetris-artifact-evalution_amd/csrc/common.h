@@ -116,10 +116,10 @@ struct tetris_g950 {
   int64_t n_entries = 0, nnz = 0;
   int32_t* d_grp_off = nullptr;   // [groups*stages+1] entry index, multiples of 8
   int32_t* d_grp_nnz = nullptr;   // [groups*stages]
-  int32_t* d_position = nullptr;  // [n_entries] s | r<<3 | ic_local<<6 | lane<<24
+  int32_t* d_position = nullptr;  // [n_entries] s | r<<3 | ic_local<<6 | slot-in-group<<24
   float* d_values = nullptr;      // [n_entries]
   int32_t* d_oc_order = nullptr;  // [slots], -1 for padding slots
-  // (LDS byte offset | accumulator index << 24, value) pairs for one tile geometry, made on first use
+  // (LDS byte offset | accumulator index << 16 | 0xC << 28, value) pairs for one tile geometry, made on first use
   std::map<tetris::BoundKey, int2*> bound;
   std::vector<tetris::Plan> plans;  // few per pack; searched linearly, most recent first
   std::mutex mu;
