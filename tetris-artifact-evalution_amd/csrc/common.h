@@ -31,7 +31,10 @@ constexpr int kBatch = 8;        // entries per 64-byte scalar fetch; every stre
 constexpr int kRefLanes = 32;    // the reference layout's lane count (Tetris/spconv2d_utils.h:15)
 constexpr int kMaxKs = 7;        // 3-bit row/column fields of the position word
 constexpr int kSlotPad = 128;    // output-channel slots are padded to a multiple of this
-constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (all regions)
+constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (all regions), single-buffered kernel
+constexpr int kBufBytes = 54272;   // one LDS buffer of the triple-buffered kernel (8-wave workgroups, 3 * 53 KiB)
+constexpr int kBufs = 3;
+constexpr int kMaxChunks = 6;      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
 constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4 * quads
 constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
 
@@ -78,6 +81,10 @@ struct Geom {
   int slots_per_unit;  // nb*ih*stride*ng
   int fill_slots;      // nq*slots_per_unit
   int spt, cg, fill_iters;
+  // triple-buffered kernel (ver == 3): a staged channel of the whole unit group is cut into 64-dword chunks,
+  // `cpp` per (unit, image) plane, and wave w fills chunks w, w + waves, ... with loads that write LDS directly
+  int ver;             // 2: single LDS tile, register staging; 3: three LDS buffers, direct-to-LDS staging
+  int cpp, nchunks, ni;
 };
 
 // Byte offset that the packed entry (ic_local, r, s) adds to a lane's LDS base address.

@@ -11,24 +11,39 @@ One *entry* of a wave's stream is two dwords {code, weight}:
                  "index the destination and the addend" enables (M0[15:12]) of VGPR index mode
 Eight entries (64 bytes) are one scalar fetch.
 
-Register plan (the kernel confines the compiler below FIRST_RESERVED):
-    v128..v255               accumulators
+Register plan (the kernel confines the compiler below A0):
+    v[ACC0 .. ACC0+NACC-1]   accumulators (v128..v255, or v64..v127 in the 64-accumulator variant)
     v[X0 + 4*NQ*b ...]       landing buffer b of the LDS reads (NBUF buffers, reads run NBUF-1 entries ahead)
     v[A0 .. A0+7]            LDS addresses of the eight entries of the batch being read
     s36..s51 / s52..s67      current / next batch, s70 = 0xC000 (index 0 + enables), s72:s73 stream address
+
+Variants (macro suffix): ""  one 64 KiB LDS tile, 128 accumulators, 16-bit LDS addresses;
+                         "3" three LDS buffers (addresses up to 160 KiB), 128 accumulators;
+                         "4" three LDS buffers, 64 accumulators and at most 64 VGPRs below them, so that four
+                             waves fit a SIMD (measured: 56 TFLOP/s for the loop alone against 43-50 with two).
 
 Per entry the loop issues: NQ ds_read_b128, one s_lshr (M0), one s_waitcnt, 4*NQ v_fma; per batch: one
 s_load_dwordx16, eight v_add_u16 (addresses), a handful of scalar ops.
 """
 
-ACC0 = 128
+TILE_BYTES = 65536   # LDS tile of the single-buffered kernel
+BUF_BYTES = 54272    # one of the three LDS buffers of the triple-buffered kernels (3 * 53 KiB <= 160 KiB)
+
+VARIANTS = {
+    "": dict(wide=False, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}),
+    "3": dict(wide=True, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}),
+    "4": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}),
+}
 
 
-def cfg(nq):
-    nbuf = {1: 4, 2: 4, 4: 2}[nq]
+def cfg(nq, variant=""):
+    """wide: LDS addresses may exceed 64 KiB (triple-buffered kernels), so they are formed in 32 bits."""
+    v = VARIANTS[variant]
+    nbuf = v["nbuf"][nq]
     x_regs = 4 * nq * nbuf
-    a0 = 128 - x_regs - 8
-    return dict(nq=nq, nbuf=nbuf, a0=a0, x0=a0 + 8, ahead=nbuf - 1, region=65536 // nq)
+    a0 = v["acc0"] - x_regs - 8
+    return dict(nq=nq, nbuf=nbuf, a0=a0, x0=a0 + 8, ahead=nbuf - 1, wide=v["wide"], acc0=v["acc0"], nacc=v["nacc"],
+                region=(BUF_BYTES if v["wide"] else TILE_BYTES) // nq)
 
 
 def reads(c, buf, addr_reg):
@@ -43,20 +58,23 @@ def reads(c, buf, addr_reg):
 def fmas(c, buf, wreg):
     out = []
     for i in range(4 * c["nq"]):
-        out.append("v_fma_f32 v%d, s%d, v%d, v%d" % (ACC0 + i, wreg, c["x0"] + 4 * c["nq"] * buf + i, ACC0 + i))
+        out.append("v_fma_f32 v%d, s%d, v%d, v%d" % (c["acc0"] + i, wreg, c["x0"] + 4 * c["nq"] * buf + i, c["acc0"] + i))
     return out
 
 
 def addresses(c, first_code_reg):
-    # under index 0: v[A0+e] (16 bit) = code[15:0] + lane base
+    # under index 0: v[A0+e] = code[15:0] + lane base (a 16-bit add, or u16 * 1 + u32 when the base can exceed 16 bits)
     out = ["s_mov_b32 m0, s70"]
     for e in range(8):
-        out.append("v_add_u16 v%d, s%d, %%[base]" % (c["a0"] + e, first_code_reg + 2 * e))
+        if c["wide"]:
+            out.append("v_mad_u32_u16 v%d, s%d, 1, %%[base]" % (c["a0"] + e, first_code_reg + 2 * e))
+        else:
+            out.append("v_add_u16 v%d, s%d, %%[base]" % (c["a0"] + e, first_code_reg + 2 * e))
     return out
 
 
-def walk(nq):
-    c = cfg(nq)
+def walk(nq, variant=""):
+    c = cfg(nq, variant)
     ahead, nbuf = c["ahead"], c["nbuf"]
     L = []
     L.append("; ---- walk one stage's stream: NQ=%d, %d landing buffers, reads %d entries ahead" % (nq, nbuf, ahead))
@@ -100,20 +118,26 @@ def walk(nq):
     return c, L
 
 
+def regs(lo, hi):
+    return ", ".join('"v%d"' % r for r in range(lo, hi))
+
+
 def main():
     print("// Generated by gen_walk_asm.py -- do not edit.")
-    for nq in (1, 2, 4):
-        c, L = walk(nq)
-        print("#define TETRIS_WALK_ASM_%d \\" % nq)
-        for line in L:
-            if line.startswith(";"):
-                continue
-            print('  "%s\\n" \\' % line)
-        print('  ""')
-        print("#define TETRIS_WALK_FIRST_RESERVED_%d %d" % (nq, c["a0"]))
-    for nq in (1, 2, 4):
-        c = cfg(nq)
-        print("#define TETRIS_WALK_VGPR_CLOBBERS_%d %s" % (nq, ", ".join('"v%d"' % r for r in range(c["a0"], 128))))
+    for variant, v in VARIANTS.items():
+        for nq in sorted(v["nbuf"]):
+            c, L = walk(nq, variant)
+            print("#define TETRIS_WALK%s_ASM_%d \\" % (variant, nq))
+            for line in L:
+                if line.startswith(";"):
+                    continue
+                print('  "%s\\n" \\' % line)
+            print('  ""')
+            print("#define TETRIS_WALK%s_FIRST_RESERVED_%d %d" % (variant, nq, c["a0"]))
+            print("#define TETRIS_WALK%s_VGPR_CLOBBERS_%d %s" % (variant, nq, regs(c["a0"], c["acc0"])))
+        print("#define TETRIS_WALK%s_ACC_CLOBBERS %s" % (variant, regs(v["acc0"], v["acc0"] + v["nacc"])))
+    print("#define TETRIS_WALK_TILE_BYTES %d" % TILE_BYTES)
+    print("#define TETRIS_WALK_BUF_BYTES %d" % BUF_BYTES)
 
 
 if __name__ == "__main__":

@@ -87,14 +87,16 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     return fail(TETRIS_EINVAL, "bad tile: lanes_w=%d quads=%d", t.lanes_w, g.nq);
   if (t.oc_per_wave != p->g)
     return fail(TETRIS_EINVAL, "tile wants %d output channels per wave, the pack was made for %d", t.oc_per_wave, p->g);
-  if (g.g * 4 * g.nq > kAccRegs)
+  if (t.waves != 1 && t.waves != 2 && t.waves != 4 && t.waves != 8 && t.waves != 16)
+    return fail(TETRIS_EINVAL, "bad tile: waves=%d (1, 2, 4, 8 or 16)", t.waves);
+  const int acc_regs = t.waves == 16 ? kAccRegs / 2 : kAccRegs;  // 16-wave workgroups run four waves per SIMD
+  if (g.g * 4 * g.nq > acc_regs)
     return fail(TETRIS_EINVAL, "oc_per_wave * 4 * quads = %d exceeds the %d accumulators of a wave", g.g * 4 * g.nq,
-                kAccRegs);
-  if (t.waves != 1 && t.waves != 2 && t.waves != 4 && t.waves != 8)
-    return fail(TETRIS_EINVAL, "bad tile: waves=%d (1, 2, 4 or 8)", t.waves);
+                acc_regs);
   const Shape s = unit_shape(t.lanes_w, g.OH, N, p->ks, stride);
   g.lw = s.lw; g.lr = s.lr; g.lh = s.lh; g.thi = s.thi; g.nb = s.nb; g.ng = s.ng; g.par = s.par; g.ih = s.ih;
-  g.region = kTileBytes / g.nq;
+  g.ver = t.waves >= 8 ? 3 : 2;
+  g.region = (g.ver == 3 ? kBufBytes : kTileBytes) / g.nq;
   g.pitch = s.pitch;
   g.plane = g.ih * g.pitch;
   g.img_stride = image_stride(s, g.tile_ic, stride);
@@ -120,6 +122,17 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   g.slots_per_unit = g.nb * g.ih * stride * g.ng;
   g.fill_slots = g.nq * g.slots_per_unit;
   const int threads = t.waves * 64;
+  if (g.ver == 3) {
+    g.cpp = ceil_div(g.plane, 64);
+    g.nchunks = g.nq * g.nb * g.cpp;
+    g.ni = ceil_div(g.nchunks, t.waves);
+    g.spt = 1; g.cg = 1; g.fill_iters = 1;
+    if (g.ni > kMaxChunks)
+      return fail(TETRIS_EINVAL, "a staged channel takes %d LDS chunks per wave (limit %d): use fewer quads or a narrower "
+                  "tile", g.ni, kMaxChunks);
+    *out = g;
+    return TETRIS_OK;
+  }
   if (g.fill_slots <= threads) {
     g.spt = 1;
     g.cg = std::min(threads / g.fill_slots, g.tile_ic);
@@ -140,16 +153,23 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
 
 // Largest tile_ic (a power of two, or C itself when smaller) that a tile shape can stage.
 static int max_tile_ic(const Shape& s, int nq, int waves, int stride, int C) {
-  const int region = kTileBytes / nq;
+  const bool v3 = waves >= 8;
+  const int region = (v3 ? kBufBytes : kTileBytes) / nq;
   const int threads = waves * 64;
   const int fill_slots = nq * s.nb * s.ih * stride * s.ng;
-  if (fill_slots > 2 * threads) return 0;
+  if (v3) {
+    if (ceil_div(nq * s.nb * ceil_div(s.ih * s.pitch, 64), waves) > kMaxChunks) return 0;
+  } else if (fill_slots > 2 * threads) {
+    return 0;
+  }
   int best = 0;
   for (int t = 1; t <= 256; t *= 2) {
     const int tic = std::min(t, C);
     if (4ll * s.nb * image_stride(s, tic, stride) > region) break;
-    int spt, cg;
-    if (fill_slots <= threads) { spt = 1; cg = std::min(threads / fill_slots, tic); } else { spt = 2; cg = 1; }
+    int spt = 1, cg = tic;
+    if (!v3) {
+      if (fill_slots <= threads) { spt = 1; cg = std::min(threads / fill_slots, tic); } else { spt = 2; cg = 1; }
+    }
     if (spt * ceil_div(tic, cg) > kFillItems) break;
     best = tic;
     if (tic == C) break;
@@ -168,7 +188,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
   //   cycles of barriers and stream start-up plus 60 per 16-byte slot a thread stages, and the waves of a
   //   workgroup wait for the slowest one at every stage; a CU holds eight waves.
   static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}};
-  static const int kWaves[] = {8, 4, 2, 1};
+  static const int kWaves[] = {16, 8, 4, 2, 1};
   const double density = 0.15;  // the mask is not known here; typical of the pruned layers this runs
   std::vector<std::pair<double, tetris_tile>> scored;
   for (int lw = 1; lw <= 62; ++lw) {
@@ -181,6 +201,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
       for (int waves : kWaves) {
         const int kb = waves * g;
         if (kb > kSlotPad) continue;
+        if (waves == 16 && (g * 4 * nq > kAccRegs / 2 || nq > 2)) continue;
         const int tic_max = max_tile_ic(s, nq, waves, stride, C);
         if (tic_max <= 0) continue;
         for (int tic = tic_max, tries = 0; tic >= 1 && tries < 3; tic /= 2, ++tries) {  // fewer channels, more stages
@@ -191,9 +212,11 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
         // waves of a workgroup meet at a barrier every stage: the slowest of them sets the pace
         const double straggle = waves > 1 ? 1.4 * std::sqrt(entries) : 0.0;
         const double items = (double)tic * nq * s.nb * s.ih * stride * s.ng / (waves * 64);  // staged slots per thread
-        const double per_wave = stages * ((entries + straggle) * (35.0 + 41.0 * nq) + 2000.0 + 60.0 * items);
+        // cycles per entry: two waves per SIMD, or four (16-wave workgroups: 110 and 180 measured for one and two quads)
+        const double per_entry = waves == 16 ? 40.0 + 70.0 * nq : 35.0 + 41.0 * nq;
+        const double per_wave = stages * ((entries + straggle) * per_entry + 2000.0 + 60.0 * items);
         const double waves_total = (double)ugroups * kblocks * waves;
-        const double rounds = waves_total / (256.0 * 8.0);
+        const double rounds = waves_total / (256.0 * (waves == 16 ? 16.0 : 8.0));
         // input re-read by every channel block, in units of the per-wave cycle count (a weak tie-breaker)
         const double reread = 1.0 + 0.02 * kblocks;
         const double cost = per_wave * std::max(rounds, 0.62) * reread;
