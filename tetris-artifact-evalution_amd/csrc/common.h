@@ -34,7 +34,7 @@ constexpr int kSlotPad = 128;    // output-channel slots are padded to a multipl
 constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (all regions), single-buffered kernel
 constexpr int kBufBytes = 54272;   // one LDS buffer of the triple-buffered kernel (8-wave workgroups, 3 * 53 KiB)
 constexpr int kBufs = 3;
-constexpr int kMaxChunks = 6;      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
+constexpr int kMaxChunks = 8;      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
 constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4 * quads
 constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
 
@@ -85,6 +85,7 @@ struct Geom {
   // `cpp` per (unit, image) plane, and wave w fills chunks w, w + waves, ... with loads that write LDS directly
   int ver;             // 2: single LDS tile, register staging; 3: three LDS buffers, direct-to-LDS staging
   int cpp, nchunks, ni;
+  int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
 };
 
 // Byte offset that the packed entry (ic_local, r, s) adds to a lane's LDS base address.

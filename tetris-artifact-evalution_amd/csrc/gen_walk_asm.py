@@ -63,47 +63,59 @@ def fmas(c, buf, wreg):
 
 
 def addresses(c, first_code_reg):
-    # under index 0: v[A0+e] = code[15:0] + lane base (a 16-bit add, or u16 * 1 + u32 when the base can exceed 16 bits)
+    # under index 0: v[A0+r] = code[15:0] of record r's first entry + lane base (a 16-bit add, or u16 * 1 + u32
+    # when the base can exceed 16 bits)
     out = ["s_mov_b32 m0, s70"]
-    for e in range(8):
+    for r in range(8 // c["share"]):
+        src = first_code_reg + 2 * r * c["share"]
         if c["wide"]:
-            out.append("v_mad_u32_u16 v%d, s%d, 1, %%[base]" % (c["a0"] + e, first_code_reg + 2 * e))
+            out.append("v_mad_u32_u16 v%d, s%d, 1, %%[base]" % (c["a0"] + r, src))
         else:
-            out.append("v_add_u16 v%d, s%d, %%[base]" % (c["a0"] + e, first_code_reg + 2 * e))
+            out.append("v_add_u16 v%d, s%d, %%[base]" % (c["a0"] + r, src))
     return out
 
 
-def walk(nq, variant=""):
+def walk(nq, variant="", share=1):
+    """share: consecutive entries of the stream come in records of `share` entries that have the same LDS offset
+    (the same input position, different output channels), so one set of LDS reads serves `share` entries."""
     c = cfg(nq, variant)
-    ahead, nbuf = c["ahead"], c["nbuf"]
+    c["share"] = share
+    R = 8 // share                       # records per batch
+    nbuf = min(c["nbuf"], R)
+    ahead = nbuf - 1                     # records of look-ahead
     L = []
-    L.append("; ---- walk one stage's stream: NQ=%d, %d landing buffers, reads %d entries ahead" % (nq, nbuf, ahead))
     for i in range(8):
         L.append("s_mov_b64 s[%d:%d], %%[c%d]" % (36 + 2 * i, 37 + 2 * i, i))
     L.append("s_mov_b32 s72, %[plo]")
     L.append("s_mov_b32 s73, %[phi]")
     L.append("s_mov_b32 s70, 0xc000")
-    for e in range(8):
-        L.append("v_mov_b32 v%d, 0" % (c["a0"] + e))
+    for r in range(R):
+        L.append("v_mov_b32 v%d, 0" % (c["a0"] + r))
     L.append("s_set_gpr_idx_on s70, 0xc")
     L += addresses(c, 36)
-    for e in range(ahead):  # prime the pipeline
-        L += reads(c, e % nbuf, c["a0"] + e)
+    for r in range(ahead):  # prime the pipeline
+        L += reads(c, r % nbuf, c["a0"] + r)
     L.append("1:")
-    L.append("s_load_dwordx16 s[52:67], s[72:73], 0x0")  # the batch after this one (may belong to the next stage)
+    L.append("s_load_dwordx16 s[52:67], s[72:73], 0x0")  # the batch after this one (may belong to the next stream)
     L.append("s_add_u32 s72, s72, 64")
     L.append("s_addc_u32 s73, s73, 0")
-    refill_at = 8 - ahead  # first step whose look-ahead entry lies in the next batch
-    for e in range(8):
-        if e == refill_at:
-            # the next batch must have arrived; its eight addresses replace the ones all consumed by now
+    refill_at = R - ahead  # first record whose look-ahead record lies in the next batch
+    for r in range(R):
+        if r == refill_at:
+            # the next batch must have arrived; its addresses replace the ones all consumed by now
             L.append("s_waitcnt lgkmcnt(0)")
             L += addresses(c, 52)
-        la = e + ahead  # entry whose reads are issued now
-        L += reads(c, la % nbuf, c["a0"] + (la % 8))
-        L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
-        L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
-        L += fmas(c, e % nbuf, 37 + 2 * e)
+        la = r + ahead  # record whose reads are issued now
+        L += reads(c, la % nbuf, c["a0"] + (la % R))
+        for k in range(share):
+            e = r * share + k
+            L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
+            if k == 0:
+                L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
+            L += fmas(c, r % nbuf, 37 + 2 * e)
+    if refill_at == R:  # no look-ahead: the next batch's addresses are formed at the end of this one
+        L.append("s_waitcnt lgkmcnt(0)")
+        L += addresses(c, 52)
     for i in range(8):
         L.append("s_mov_b64 s[%d:%d], s[%d:%d]" % (36 + 2 * i, 37 + 2 * i, 52 + 2 * i, 53 + 2 * i))
     L.append("s_sub_u32 %[nb], %[nb], 1")
@@ -126,13 +138,12 @@ def main():
     print("// Generated by gen_walk_asm.py -- do not edit.")
     for variant, v in VARIANTS.items():
         for nq in sorted(v["nbuf"]):
-            c, L = walk(nq, variant)
-            print("#define TETRIS_WALK%s_ASM_%d \\" % (variant, nq))
-            for line in L:
-                if line.startswith(";"):
-                    continue
-                print('  "%s\\n" \\' % line)
-            print('  ""')
+            for share in (1, 2, 4):
+                c, L = walk(nq, variant, share)
+                print("#define TETRIS_WALK%s_ASM_%d_S%d \\" % (variant, nq, share))
+                for line in L:
+                    print('  "%s\\n" \\' % line)
+                print('  ""')
             print("#define TETRIS_WALK%s_FIRST_RESERVED_%d %d" % (variant, nq, c["a0"]))
             print("#define TETRIS_WALK%s_VGPR_CLOBBERS_%d %s" % (variant, nq, regs(c["a0"], c["acc0"])))
         print("#define TETRIS_WALK%s_ACC_CLOBBERS %s" % (variant, regs(v["acc0"], v["acc0"] + v["nacc"])))

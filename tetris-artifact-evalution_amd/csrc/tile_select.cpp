@@ -125,7 +125,10 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   if (g.ver == 3) {
     g.cpp = ceil_div(g.plane, 64);
     g.nchunks = g.nq * g.nb * g.cpp;
-    g.ni = ceil_div(g.nchunks, t.waves);
+    // a 16-wave workgroup leaves the staging to its four oldest waves when they can hold the plan
+    g.stagers = t.waves;
+    if (t.waves == 16) g.stagers = g.nchunks <= 4 * kMaxChunks ? 4 : g.nchunks <= 8 * kMaxChunks ? 8 : 16;
+    g.ni = ceil_div(g.nchunks, g.stagers);
     g.spt = 1; g.cg = 1; g.fill_iters = 1;
     if (g.ni > kMaxChunks)
       return fail(TETRIS_EINVAL, "a staged channel takes %d LDS chunks per wave (limit %d): use fewer quads or a narrower "
@@ -187,7 +190,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
   //   FMA is what binds it) and about 0.62 of that when it has the SIMD to itself; a stage costs about 2000
   //   cycles of barriers and stream start-up plus 60 per 16-byte slot a thread stages, and the waves of a
   //   workgroup wait for the slowest one at every stage; a CU holds eight waves.
-  static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}};
+  static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}, {2, 4}, {1, 4}};
   static const int kWaves[] = {16, 8, 4, 2, 1};
   const double density = 0.15;  // the mask is not known here; typical of the pruned layers this runs
   std::vector<std::pair<double, tetris_tile>> scored;
