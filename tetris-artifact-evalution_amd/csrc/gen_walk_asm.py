@@ -95,32 +95,44 @@ def walk(nq, variant="", share=1):
     L += addresses(c, 36)
     for r in range(ahead):  # prime the pipeline
         L += reads(c, r % nbuf, c["a0"] + r)
-    L.append("1:")
-    L.append("s_load_dwordx16 s[52:67], s[72:73], 0x0")  # the batch after this one (may belong to the next stream)
-    L.append("s_add_u32 s72, s72, 64")
-    L.append("s_addc_u32 s73, s73, 0")
-    refill_at = R - ahead  # first record whose look-ahead record lies in the next batch
-    for r in range(R):
-        if r == refill_at:
-            # the next batch must have arrived; its addresses replace the ones all consumed by now
-            L.append("s_waitcnt lgkmcnt(0)")
-            L += addresses(c, 52)
-        la = r + ahead  # record whose reads are issued now
-        L += reads(c, la % nbuf, c["a0"] + (la % R))
-        for k in range(share):
-            e = r * share + k
-            L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
-            if k == 0:
-                L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
-            L += fmas(c, r % nbuf, 37 + 2 * e)
-    if refill_at == R:  # no look-ahead: the next batch's addresses are formed at the end of this one
-        L.append("s_waitcnt lgkmcnt(0)")
-        L += addresses(c, 52)
-    for i in range(8):
-        L.append("s_mov_b64 s[%d:%d], s[%d:%d]" % (36 + 2 * i, 37 + 2 * i, 52 + 2 * i, 53 + 2 * i))
-    L.append("s_sub_u32 %[nb], %[nb], 1")
-    L.append("s_cmp_lg_u32 %[nb], 0")
-    L.append("s_cbranch_scc1 1b")
+    # The loop body handles one batch and is unrolled four times; copy k runs at wave priority k.  A wave enters at
+    # copy %[ph] (its index on the SIMD plus a running count), so the waves of a SIMD hold different priorities
+    # that rotate with every batch.  Left alone the SIMD serves its oldest wave first: that wave finishes its stage
+    # early and idles at the barrier while the youngest runs the tail of the stage alone, too slowly to fill the
+    # SIMD by itself.
+    for k in (1, 2, 3):
+        L.append("s_cmp_eq_u32 %%[ph], %d" % k)
+        L.append("s_cbranch_scc1 %df" % (k + 1))
+    for k in range(4):
+        L.append("%d:" % (k + 1))
+        L.append("s_setprio %d" % k)
+        L.append("s_load_dwordx16 s[52:67], s[72:73], 0x0")  # the batch after this one (may belong to the next stream)
+        L.append("s_add_u32 s72, s72, 64")
+        L.append("s_addc_u32 s73, s73, 0")
+        refill_at = R - ahead  # first record whose look-ahead record lies in the next batch
+        for r in range(R):
+            if r == refill_at:
+                # the next batch must have arrived; its addresses replace the ones all consumed by now
+                L.append("s_waitcnt lgkmcnt(0)")
+                L += addresses(c, 52)
+            la = r + ahead  # record whose reads are issued now
+            L += reads(c, la % nbuf, c["a0"] + (la % R))
+            for kk in range(share):
+                e = r * share + kk
+                L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
+                if kk == 0:
+                    L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
+                L += fmas(c, r % nbuf, 37 + 2 * e)
+        for i in range(8):
+            L.append("s_mov_b64 s[%d:%d], s[%d:%d]" % (36 + 2 * i, 37 + 2 * i, 52 + 2 * i, 53 + 2 * i))
+        L.append("s_sub_u32 %[nb], %[nb], 1")
+        L.append("s_cmp_lg_u32 %[nb], 0")
+        if k < 3:
+            L.append("s_cbranch_scc0 9f")
+        else:
+            L.append("s_cbranch_scc1 1b")
+    L.append("9:")
+    L.append("s_setprio 3")  # what follows a walk (issuing the staging loads, reaching the barrier) should not wait
     L.append("s_waitcnt lgkmcnt(0)")  # drain the look-ahead reads (their data is not used)
     L.append("s_set_gpr_idx_off")
     for i in range(8):
