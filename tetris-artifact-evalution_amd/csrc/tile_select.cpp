@@ -118,6 +118,9 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   if (img_bytes * ((long long)g.nq * g.nb + 2) >= (1ll << 31))
     return fail(TETRIS_EINVAL, "images too large for the 2 GB input window of a workgroup");
   if ((long long)N * p->K * g.OH * g.OW >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
+  // ... and writes its outputs through one as well
+  if (4ll * p->K * g.OH * g.OW * ((long long)g.nq * g.nb + 2) >= (1ll << 31))
+    return fail(TETRIS_EINVAL, "images too large for the 2 GB output window of a workgroup");
   // staging plan
   g.slots_per_unit = g.nb * g.ih * stride * g.ng;
   g.fill_slots = g.nq * g.slots_per_unit;
