@@ -38,9 +38,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
     ap.add_argument("--layer-repeat", type=int, default=30, help="timed launches per layer for the per-layer table")
-    ap.add_argument("--tile", choices=("autotune", "select"), default="autotune",
-                    help="autotune: time the selector's best candidates per layer during set-up (what the reference's "
-                         "driver does with its 185-entry table); select: take the selector's first choice unmeasured")
+    ap.add_argument("--tile", choices=("autotune", "select"), default="select",
+                    help="select: the library's own choice (its built-in table of tiles measured on MI355X, else its cycle "
+                         "model); autotune: time the model's best candidates per layer during set-up, as the reference's "
+                         "driver does with its 185-entry table")
     ap.add_argument("--candidates", type=int, default=24)
     ap.add_argument("--save-tiles", metavar="FILE", help="write the tile chosen for every layer to FILE (JSON)")
     ap.add_argument("--load-tiles", metavar="FILE", help="use the tiles a previous --save-tiles run wrote (so that a "

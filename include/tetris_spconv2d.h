@@ -110,13 +110,15 @@ typedef struct tetris_tile {
   int32_t tile_ic;     /* input channels staged in LDS at a time                                   */
 } tetris_tile;
 
+/* Unmeasured selection: a built-in table of tiles measured on MI355X for the layer shapes of the benchmark
+ * suites (csrc/tuned_tiles.inc, made by tetris_amd/tune.py), else the first choice of a cycle model. */
 int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_channel, int kernel_size, int stride,
                        int padding, tetris_tile* out);
 
 /* Measured selection, the counterpart of GetTetrisSparseConv2dTime (Tetris/spconv2d.cc:72-329): packs the filter
  * for the `max_candidates` (0 = 24) tile shapes the model of tetris_tile_select ranks best, times each on the
- * device with the real weights (1 warm-up + 3 launches on zero-filled input) and returns the fastest and its
- * milliseconds per launch.  Allocates and frees its own device buffers; synchronises `stream`. */
+ * device with the real weights (1 warm-up + 3 launches on zero-filled input), times the four fastest again
+ * (2 + 10 launches) and returns the fastest and its milliseconds per launch.  Allocates and frees its own device buffers; synchronises `stream`. */
 int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int img_w, int in_channel, int out_channel,
                          int kernel_size, int stride, int padding, int max_candidates, void* stream,
                          tetris_tile* out, float* ms_out);

@@ -6,6 +6,8 @@
 #include <cstring>
 #include <fstream>
 
+#include <algorithm>
+
 #include "common.h"
 
 namespace tetris {
@@ -299,11 +301,10 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
   HIPA(hipMemsetAsync(d_in, 0, in_bytes, stream));  // timing does not depend on the values
   HIPA(hipMemcpyAsync(d_f, h_filter, f_bytes, hipMemcpyHostToDevice, stream));
 #undef HIPA
-  float best_ms = 1e30f;
-  tetris_tile best = ranked[0];
-  int tried = 0;
+  // first pass: a quick look at every candidate; second pass: the four fastest again, with more launches
+  std::vector<std::pair<float, tetris_tile>> timed;
   for (const tetris_tile& t : ranked) {
-    if (tried >= max_candidates) break;
+    if ((int)timed.size() >= max_candidates) break;
     const std::pair<int, int> key(t.tile_ic, t.oc_per_wave);
     auto it = packs.find(key);
     if (it == packs.end()) {
@@ -316,13 +317,24 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
     rc = time_launches(it->second, d_in, d_out, N, H, W, stride, pad, &t, stream, 1, 3, &ms);
     if (rc == TETRIS_EINVAL) continue;  // the model ranks shapes make_geom may still refuse
     if (rc) return done(rc);
-    ++tried;
+    timed.emplace_back(ms, t);
+  }
+  if (timed.empty()) return done(fail(TETRIS_EINVAL, "no tile shape could be launched for this layer"));
+  std::stable_sort(timed.begin(), timed.end(),
+                   [](const std::pair<float, tetris_tile>& a, const std::pair<float, tetris_tile>& b) { return a.first < b.first; });
+  float best_ms = 1e30f;
+  tetris_tile best = timed[0].second;
+  for (size_t i = 0; i < timed.size() && i < 4; ++i) {
+    const tetris_tile& t = timed[i].second;
+    float ms = 0;
+    rc = time_launches(packs[std::make_pair(t.tile_ic, t.oc_per_wave)], d_in, d_out, N, H, W, stride, pad, &t, stream, 2,
+                       10, &ms);
+    if (rc) return done(rc);
     if (ms < best_ms) {
       best_ms = ms;
       best = t;
     }
   }
-  if (tried == 0) return done(fail(TETRIS_EINVAL, "no tile shape could be launched for this layer"));
   *out = best;
   if (ms_out) *ms_out = best_ms;
   return done(TETRIS_OK);

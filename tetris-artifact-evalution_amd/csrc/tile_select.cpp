@@ -241,7 +241,33 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
   return TETRIS_OK;
 }
 
+namespace {
+// Tiles measured on MI355X (tetris_tile_autotune over the benchmark suites), keyed by layer shape.  They play the
+// part of the reference's per-layer table of template instantiations (Tetris/spconv2d.cc:90-329).
+struct Tuned {
+  int N, H, W, C, K, ks, stride, pad;
+  tetris_tile tile;
+};
+const Tuned kTuned[] = {
+#include "tuned_tiles.inc"
+    {0, 0, 0, 0, 0, 0, 0, 0, {0, 0, 0, 0, 0}}};
+}  // namespace
+
 int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t) {
+  for (const Tuned& e : kTuned)
+    if (e.N == N && e.H == H && e.W == W && e.C == C && e.K == K && e.ks == ks && e.stride == stride && e.pad == pad) {
+      // trust the table only as far as the kernel's own checks go
+      tetris_g950 shape;
+      shape.C = C; shape.K = K; shape.ks = ks; shape.tile_ic = e.tile.tile_ic; shape.g = e.tile.oc_per_wave;
+      shape.stages = ceil_div(C, e.tile.tile_ic);
+      shape.slots = ceil_div(K, kSlotPad) * kSlotPad;
+      Geom g;
+      if (make_geom(&shape, N, H, W, stride, pad, e.tile, &g) == TETRIS_OK) {
+        *t = e.tile;
+        return TETRIS_OK;
+      }
+      break;
+    }
   std::vector<tetris_tile> ranked;
   const int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked);
   if (rc) return rc;
