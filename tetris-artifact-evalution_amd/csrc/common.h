@@ -34,12 +34,15 @@ constexpr int kSlotPad = 128;    // output-channel slots are padded to a multipl
 constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (all regions), single-buffered kernel
 constexpr int kBufBytes = 54272;   // one LDS buffer of the triple-buffered kernel (8-wave workgroups, 3 * 53 KiB)
 constexpr int kBufs = 3;
-constexpr int kMaxChunks = 8;      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
+constexpr int kMaxChunks = 8;      // (6 in a 16-wave workgroup, whose waves have fewer registers)
+constexpr int kMaxChunks16 = 6;
+//      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
 constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4 * quads
 constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
 
 inline int out_extent(int in, int pad, int ks, int stride) { return (in + 2 * pad - ks) / stride + 1; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline unsigned magic_reciprocal(int d) { return d <= 1 ? 0u : (unsigned)((1ull << 32) / (unsigned)d) + 1u; }
 
 // ---- kernel geometry --------------------------------------------------------------------------
 // Output pixels are cut into *units* of up to 64 quads: a unit is `lh` virtual rows by 4*lw columns, lane
@@ -86,6 +89,8 @@ struct Geom {
   int ver;             // 2: single LDS tile, register staging; 3: three LDS buffers, direct-to-LDS staging
   int cpp, nchunks, ni;
   int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
+  // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
+  unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi;
 };
 
 // Byte offset that the packed entry (ic_local, r, s) adds to a lane's LDS base address.

@@ -125,17 +125,33 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   g.slots_per_unit = g.nb * g.ih * stride * g.ng;
   g.fill_slots = g.nq * g.slots_per_unit;
   const int threads = t.waves * 64;
+  {
+    // the kernels divide by these with a multiply-high, exact while dividend * divisor < 2^32
+    const long long upi = (long long)g.units_w * g.units_h;
+    if (units * upi >= (1ll << 32)) return fail(TETRIS_EINVAL, "too many pixel units for the kernel's index arithmetic");
+    g.m_upi = magic_reciprocal((int)upi);
+    g.m_units_w = magic_reciprocal(g.units_w);
+    g.m_lr = magic_reciprocal(g.lr);
+    g.m_thi = magic_reciprocal(g.thi);
+  }
   if (g.ver == 3) {
     g.cpp = ceil_div(g.plane, 64);
     g.nchunks = g.nq * g.nb * g.cpp;
     // a 16-wave workgroup leaves the staging to its four oldest waves when they can hold the plan
     g.stagers = t.waves;
-    if (t.waves == 16) g.stagers = g.nchunks <= 4 * kMaxChunks ? 4 : g.nchunks <= 8 * kMaxChunks ? 8 : 16;
+    const int max_chunks = t.waves == 16 ? kMaxChunks16 : kMaxChunks;
+    if (t.waves == 16) g.stagers = g.nchunks <= 4 * max_chunks ? 4 : g.nchunks <= 8 * max_chunks ? 8 : 16;
     g.ni = ceil_div(g.nchunks, g.stagers);
+    if (64ll * (g.cpp + 1) * g.pitch >= (1ll << 32))
+      return fail(TETRIS_EINVAL, "too many pixel units for the kernel's index arithmetic");
+    g.m_per_unit = magic_reciprocal(g.nb * g.cpp);
+    g.m_cpp = magic_reciprocal(g.cpp);
+    g.m_pitch = magic_reciprocal(g.pitch);
+    g.m_par = magic_reciprocal(g.par);
     g.spt = 1; g.cg = 1; g.fill_iters = 1;
-    if (g.ni > kMaxChunks)
+    if (g.ni > max_chunks)
       return fail(TETRIS_EINVAL, "a staged channel takes %d LDS chunks per wave (limit %d): use fewer quads or a narrower "
-                  "tile", g.ni, kMaxChunks);
+                  "tile", g.ni, max_chunks);
     *out = g;
     return TETRIS_OK;
   }
@@ -164,7 +180,7 @@ static int max_tile_ic(const Shape& s, int nq, int waves, int stride, int C) {
   const int threads = waves * 64;
   const int fill_slots = nq * s.nb * s.ih * stride * s.ng;
   if (v3) {
-    if (ceil_div(nq * s.nb * ceil_div(s.ih * s.pitch, 64), waves) > kMaxChunks) return 0;
+    if (ceil_div(nq * s.nb * ceil_div(s.ih * s.pitch, 64), waves) > (waves == 16 ? kMaxChunks16 : kMaxChunks)) return 0;
   } else if (fill_slots > 2 * threads) {
     return 0;
   }
