@@ -90,7 +90,8 @@ struct Geom {
   int cpp, nchunks, ni;
   int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
-  unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi;
+  unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks;
+  unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan
 };
 
 // Byte offset that the packed entry (ic_local, r, s) adds to a lane's LDS base address.

@@ -133,6 +133,8 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     g.m_units_w = magic_reciprocal(g.units_w);
     g.m_lr = magic_reciprocal(g.lr);
     g.m_thi = magic_reciprocal(g.thi);
+    if ((long long)g.ugroups * g.kblocks * g.kblocks >= (1ll << 32)) return fail(TETRIS_EINVAL, "grid too large");
+    g.m_kblocks = magic_reciprocal(g.kblocks);
   }
   if (g.ver == 3) {
     g.cpp = ceil_div(g.plane, 64);
@@ -155,6 +157,11 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     *out = g;
     return TETRIS_OK;
   }
+  g.m_fill_slots = magic_reciprocal(g.fill_slots);
+  g.m_slots_per_unit = magic_reciprocal(g.slots_per_unit);
+  g.m_per_img = magic_reciprocal(g.ih * stride * g.ng);
+  g.m_per_row = magic_reciprocal(stride * g.ng);
+  g.m_ng = magic_reciprocal(g.ng);
   if (g.fill_slots <= threads) {
     g.spt = 1;
     g.cg = std::min(threads / g.fill_slots, g.tile_ic);
