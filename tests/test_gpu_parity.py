@@ -79,7 +79,8 @@ TILES = [  # lanes_w, quads, oc_per_wave, waves
     (16, 4, 8, 8), (16, 2, 16, 8), (16, 1, 32, 8), (8, 2, 16, 8), (4, 4, 8, 8), (2, 2, 8, 8), (14, 2, 16, 8),
     (7, 4, 4, 8), (13, 1, 16, 8), (16, 2, 8, 4), (8, 1, 32, 4), (16, 1, 8, 2), (1, 2, 16, 8), (5, 4, 8, 8),
     (16, 1, 16, 1), (3, 1, 32, 8),
-    (16, 2, 8, 16), (14, 2, 8, 16), (7, 1, 16, 16), (4, 1, 8, 16), (8, 2, 4, 16), (2, 1, 16, 16)]  # four waves per SIMD
+    (16, 2, 8, 16), (14, 2, 8, 16), (7, 1, 16, 16), (4, 1, 8, 16), (8, 2, 4, 16), (2, 1, 16, 16),  # four waves per SIMD
+    (14, 2, 8, 8), (7, 2, 4, 8), (8, 1, 16, 8), (3, 1, 8, 8), (16, 1, 4, 8)]  # ... as two 8-wave workgroups per CU
 
 
 @pytest.mark.parametrize("tile", TILES)

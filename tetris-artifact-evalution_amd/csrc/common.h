@@ -33,6 +33,7 @@ constexpr int kMaxKs = 7;        // 3-bit row/column fields of the position word
 constexpr int kSlotPad = 128;    // output-channel slots are padded to a multiple of this
 constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (all regions), single-buffered kernel
 constexpr int kBufBytes = 54272;   // one LDS buffer of the triple-buffered kernel (8-wave workgroups, 3 * 53 KiB)
+constexpr int kHalfBufBytes = 27136;  // ... when two 8-wave workgroups of 64-accumulator waves share a CU
 constexpr int kBufs = 3;
 constexpr int kMaxChunks = 8;      // (6 in a 16-wave workgroup, whose waves have fewer registers)
 constexpr int kMaxChunks16 = 6;
@@ -88,6 +89,7 @@ struct Geom {
   // `cpp` per (unit, image) plane, and wave w fills chunks w, w + waves, ... with loads that write LDS directly
   int ver;             // 2: single LDS tile, register staging; 3: three LDS buffers, direct-to-LDS staging
   int cpp, nchunks, ni;
+  int buf_bytes;       // size of one of the three LDS buffers: kBufBytes, or kHalfBufBytes (8 waves of <= 64 accumulators)
   int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks;

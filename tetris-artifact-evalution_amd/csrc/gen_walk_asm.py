@@ -20,7 +20,8 @@ Register plan (the kernel confines the compiler below A0):
 Variants (macro suffix): ""  one 64 KiB LDS tile, 128 accumulators, 16-bit LDS addresses;
                          "3" three LDS buffers (addresses up to 160 KiB), 128 accumulators;
                          "4" three LDS buffers, 64 accumulators and at most 64 VGPRs below them, so that four
-                             waves fit a SIMD (measured: 56 TFLOP/s for the loop alone against 43-50 with two).
+                             waves fit a SIMD (measured: 56 TFLOP/s for the loop alone against 43-50 with two);
+                         "5" as "4" with buffers of half the size, for two 8-wave workgroups per CU.
 
 Per entry the loop issues: NQ ds_read_b128, one s_lshr (M0), one s_waitcnt, 4*NQ v_fma; per batch: one
 s_load_dwordx16, eight v_add_u16 (addresses), a handful of scalar ops.
@@ -28,11 +29,16 @@ s_load_dwordx16, eight v_add_u16 (addresses), a handful of scalar ops.
 
 TILE_BYTES = 65536   # LDS tile of the single-buffered kernel
 BUF_BYTES = 54272    # one of the three LDS buffers of the triple-buffered kernels (3 * 53 KiB <= 160 KiB)
+HALF_BUF_BYTES = 27136  # ... when two workgroups share a CU
+
+# record sizes to emit loops for; the pack only makes single-entry records so far (2 and 4 measured 1.1-1.2x)
+SHARES = (1,)
 
 VARIANTS = {
     "": dict(wide=False, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}),
     "3": dict(wide=True, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}),
     "4": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}),
+    "5": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}, buf=HALF_BUF_BYTES),
 }
 
 
@@ -43,7 +49,7 @@ def cfg(nq, variant=""):
     x_regs = 4 * nq * nbuf
     a0 = v["acc0"] - x_regs - 8
     return dict(nq=nq, nbuf=nbuf, a0=a0, x0=a0 + 8, ahead=nbuf - 1, wide=v["wide"], acc0=v["acc0"], nacc=v["nacc"],
-                region=(BUF_BYTES if v["wide"] else TILE_BYTES) // nq)
+                region=(v.get("buf", BUF_BYTES) if v["wide"] else TILE_BYTES) // nq)
 
 
 def reads(c, buf, addr_reg):
@@ -150,7 +156,7 @@ def main():
     print("// Generated by gen_walk_asm.py -- do not edit.")
     for variant, v in VARIANTS.items():
         for nq in sorted(v["nbuf"]):
-            for share in (1, 2, 4):
+            for share in SHARES:
                 c, L = walk(nq, variant, share)
                 print("#define TETRIS_WALK%s_ASM_%d_S%d \\" % (variant, nq, share))
                 for line in L:
@@ -161,6 +167,7 @@ def main():
         print("#define TETRIS_WALK%s_ACC_CLOBBERS %s" % (variant, regs(v["acc0"], v["acc0"] + v["nacc"])))
     print("#define TETRIS_WALK_TILE_BYTES %d" % TILE_BYTES)
     print("#define TETRIS_WALK_BUF_BYTES %d" % BUF_BYTES)
+    print("#define TETRIS_WALK_HALF_BUF_BYTES %d" % HALF_BUF_BYTES)
 
 
 if __name__ == "__main__":

@@ -96,7 +96,9 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   const Shape s = unit_shape(t.lanes_w, g.OH, N, p->ks, stride);
   g.lw = s.lw; g.lr = s.lr; g.lh = s.lh; g.thi = s.thi; g.nb = s.nb; g.ng = s.ng; g.par = s.par; g.ih = s.ih;
   g.ver = t.waves >= 8 ? 3 : 2;
-  g.region = (g.ver == 3 ? kBufBytes : kTileBytes) / g.nq;
+  // 8 waves that need at most 64 accumulators each leave room for a second workgroup on the CU
+  g.buf_bytes = (t.waves == 8 && g.g * 4 * g.nq <= kAccRegs / 2 && g.nq <= 2) ? kHalfBufBytes : kBufBytes;
+  g.region = (g.ver == 3 ? g.buf_bytes : kTileBytes) / g.nq;
   g.pitch = s.pitch;
   g.plane = g.ih * g.pitch;
   g.img_stride = image_stride(s, g.tile_ic, stride);
@@ -141,7 +143,7 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     g.nchunks = g.nq * g.nb * g.cpp;
     // a 16-wave workgroup leaves the staging to its four oldest waves when they can hold the plan
     g.stagers = t.waves;
-    const int max_chunks = t.waves == 16 ? kMaxChunks16 : kMaxChunks;
+    const int max_chunks = (t.waves == 16 || g.buf_bytes == kHalfBufBytes) ? kMaxChunks16 : kMaxChunks;
     if (t.waves == 16) g.stagers = g.nchunks <= 4 * max_chunks ? 4 : g.nchunks <= 8 * max_chunks ? 8 : 16;
     g.ni = ceil_div(g.nchunks, g.stagers);
     if (64ll * (g.cpp + 1) * g.pitch >= (1ll << 32))
@@ -181,13 +183,14 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
 }
 
 // Largest tile_ic (a power of two, or C itself when smaller) that a tile shape can stage.
-static int max_tile_ic(const Shape& s, int nq, int waves, int stride, int C) {
+static int max_tile_ic(const Shape& s, int nq, int g, int waves, int stride, int C) {
   const bool v3 = waves >= 8;
-  const int region = (v3 ? kBufBytes : kTileBytes) / nq;
+  const bool half = waves == 8 && g * 4 * nq <= kAccRegs / 2 && nq <= 2;
+  const int region = (v3 ? (half ? kHalfBufBytes : kBufBytes) : kTileBytes) / nq;
   const int threads = waves * 64;
   const int fill_slots = nq * s.nb * s.ih * stride * s.ng;
   if (v3) {
-    if (ceil_div(nq * s.nb * ceil_div(s.ih * s.pitch, 64), waves) > (waves == 16 ? kMaxChunks16 : kMaxChunks)) return 0;
+    if (ceil_div(nq * s.nb * ceil_div(s.ih * s.pitch, 64), waves) > (waves == 16 || half ? kMaxChunks16 : kMaxChunks)) return 0;
   } else if (fill_slots > 2 * threads) {
     return 0;
   }
@@ -231,7 +234,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
         const int kb = waves * g;
         if (kb > kSlotPad) continue;
         if (waves == 16 && (g * 4 * nq > kAccRegs / 2 || nq > 2)) continue;
-        const int tic_max = max_tile_ic(s, nq, waves, stride, C);
+        const int tic_max = max_tile_ic(s, nq, g, waves, stride, C);
         if (tic_max <= 0) continue;
         for (int tic = tic_max, tries = 0; tic >= 1 && tries < 3; tic /= 2, ++tries) {  // fewer channels, more stages
         const long long ugroups = (units + nq - 1) / nq;
@@ -242,10 +245,11 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
         const double straggle = waves > 1 ? 1.4 * std::sqrt(entries) : 0.0;
         const double items = (double)tic * nq * s.nb * s.ih * stride * s.ng / (waves * 64);  // staged slots per thread
         // cycles per entry: two waves per SIMD, or four (16-wave workgroups: 110 and 180 measured for one and two quads)
-        const double per_entry = waves == 16 ? 40.0 + 70.0 * nq : 35.0 + 41.0 * nq;
+        const bool four = waves == 16 || (waves == 8 && g * 4 * nq <= kAccRegs / 2 && nq <= 2);  // waves per SIMD
+        const double per_entry = four ? 40.0 + 70.0 * nq : 35.0 + 41.0 * nq;
         const double per_wave = stages * ((entries + straggle) * per_entry + 2000.0 + 60.0 * items);
         const double waves_total = (double)ugroups * kblocks * waves;
-        const double rounds = waves_total / (256.0 * (waves == 16 ? 16.0 : 8.0));
+        const double rounds = waves_total / (256.0 * (four ? 16.0 : 8.0));
         // input re-read by every channel block, in units of the per-wave cycle count (a weak tie-breaker)
         const double reread = 1.0 + 0.02 * kblocks;
         const double cost = per_wave * std::max(rounds, 0.62) * reread;
