@@ -50,6 +50,8 @@ SHAPES = [  # N, C, H, W, K, ks, stride, pad, sparsity  -- the reference's kerne
     (1, 16, 10, 10, 24, 3, 1, 1, 1.0),   # all-zero filter
     (1, 16, 10, 10, 24, 3, 1, 1, 0.0),   # dense filter
     (17, 5, 3, 3, 260, 1, 1, 0, 0.5),    # more images than a tile folds, K over two slot paddings
+    (2, 160, 7, 7, 48, 3, 1, 1, 0.8),    # few pixels, many channels: workgroups split the channel reduction
+    (1, 300, 5, 5, 20, 1, 1, 0, 0.7),
 ]
 
 

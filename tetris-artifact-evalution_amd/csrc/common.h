@@ -90,9 +90,11 @@ struct Geom {
   int ver;             // 2: single LDS tile, register staging; 3: three LDS buffers, direct-to-LDS staging
   int cpp, nchunks, ni;
   int buf_bytes;       // size of one of the three LDS buffers: kBufBytes, or kHalfBufBytes (8 waves of <= 64 accumulators)
+  int csplit;          // workgroups that share an output tile, each reducing a slice of the stages and adding its
+                       // partial sums to the (pre-zeroed) output with atomics; 1 = plain stores
   int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
-  unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks;
+  unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan
 };
 
@@ -172,6 +174,7 @@ int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, 
 int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked);
 
 // spconv2d_kernel.hip
+// launches the conv (after a zero fill of the output when the geometry splits the channel reduction)
 int launch_conv(const Geom& g, const float* d_in, float* d_out, const int2* entries, const int32_t* grp_off,
                 const int32_t* oc_order, hipStream_t stream);
 

@@ -135,8 +135,17 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     g.m_units_w = magic_reciprocal(g.units_w);
     g.m_lr = magic_reciprocal(g.lr);
     g.m_thi = magic_reciprocal(g.thi);
-    if ((long long)g.ugroups * g.kblocks * g.kblocks >= (1ll << 32)) return fail(TETRIS_EINVAL, "grid too large");
+    // Small feature maps leave most of the 256 CUs without a workgroup: then several workgroups share an output
+    // tile, each reducing a slice of the input-channel stages (at least four stages each, at most eight slices).
+    const bool four = t.waves == 16 || g.buf_bytes == kHalfBufBytes;  // waves per SIMD the kernel variant allows
+    const long long room = 256ll * (g.ver == 3 && four ? 16 : 8);
+    const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
+    g.csplit = 1;
+    while (g.csplit < 8 && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
+    if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32))
+      return fail(TETRIS_EINVAL, "grid too large");
     g.m_kblocks = magic_reciprocal(g.kblocks);
+    g.m_csplit = magic_reciprocal(g.csplit);
   }
   if (g.ver == 3) {
     g.cpp = ceil_div(g.plane, 64);
