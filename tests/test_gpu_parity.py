@@ -247,3 +247,33 @@ def test_every_layer_shape_of_the_suites(env, suite):
         worst = max(worst, err)
         pk.close()
     assert len(seen) >= 4
+
+
+def test_random_shapes_with_library_tiles(env):
+    # Seeded random layer shapes (all kernel-size/stride families, ragged channel counts, tiny and wide images), the
+    # tile left to the library: exercises every kernel variant the selector can reach, the channel-split path included.
+    T, torch, O = env
+    rng = np.random.default_rng(2024)
+    variants = set()
+    for case in range(60):
+        ks, stride = [(1, 1), (3, 1), (3, 2), (1, 2), (5, 1), (7, 2)][int(rng.integers(6))]
+        pad = int(rng.integers(0, ks // 2 + 1)) if ks > 1 else 0
+        N = int(rng.integers(1, 6))
+        C = int(rng.choice([3, 8, 17, 32, 96, 130, 256, 520]))
+        K = int(rng.choice([4, 16, 33, 64, 128, 200, 384]))
+        H = int(rng.choice([5, 7, 13, 14, 28, 31, 56, 75]))
+        W = int(rng.choice([5, 7, 13, 14, 28, 33, 56, 90]))
+        if H + 2 * pad < ks or W + 2 * pad < ks or N * C * H * W > 6e6 or N * K * H * W * C * ks * ks > 3e10:
+            continue
+        sp = float(rng.choice([0.5, 0.8, 0.9, 0.97]))
+        w = sparse_filter(rng, K, C, ks, sp)
+        x = relu_like(rng, (N, C, H, W))
+        tile = T.tile_select(N, H, W, C, K, ks, stride, pad)
+        pk = T.G950Filter.for_tile(w, tile)
+        y = run_conv(T, torch, pk, x, K, ks, stride, pad, tile)
+        ref = O.G950Pack(w, 32, 8).conv(x, stride, pad, threads=min(16, O.max_threads()))
+        err = max_rel_err(y, ref)
+        assert err <= TOL, (case, (N, C, H, W, K, ks, stride, pad, sp), tile, err)
+        variants.add((tile.waves, tile.quads))
+        pk.close()
+    assert len(variants) >= 3, variants
