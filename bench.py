@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--save-tiles", metavar="FILE", help="write the tile chosen for every layer to FILE (JSON)")
     ap.add_argument("--load-tiles", metavar="FILE", help="use the tiles a previous --save-tiles run wrote (so that a "
                     "profiled run launches nothing but packing and the timed convolutions)")
+    ap.add_argument("--dense-baseline", action="store_true",
+                    help="also time the vendor's dense fp32 convolution (MIOpen through torch) on the same layers, as "
+                         "context (the reference compares with cuDNN the same way, Tetris/cuda_utils.cc:6-132)")
     ap.add_argument("--calibrate-copy", type=int, metavar="MIB", default=0,
                     help="instead of the benchmark, run one elementwise copy kernel over MIB MiB (reads MIB, writes MIB): "
                          "the known-size dispatch that scales the FETCH_SIZE / WRITE_SIZE counters")
@@ -210,6 +213,30 @@ def main():
                                            "unit": "GFLOP/s", "cores": 1, "kind": "reference",
                                            "sample": "single 64->128 56x56 3x3 layer, batch 1, %.2f s" % dt}
 
+    context = None
+    if args.dense_baseline:
+        import torch.nn.functional as F
+        ws = [torch.from_numpy(W.make_weights(L)).to(dev) for L in layers]
+
+        def dense_step():
+            for L, x, w in zip(layers, xs, ws):
+                F.conv2d(x, w, None, L.stride, L.pad)
+
+        for _ in range(3):
+            dense_step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            dense_step()
+        e1.record()
+        torch.cuda.synchronize()
+        dense_ms = e0.elapsed_time(e1) / args.steps
+        context = {"vendor_dense_fp32_ms_per_step": round(dense_ms, 4),
+                   "vendor_dense_fp32_gflops": round(fl_dense / (dense_ms * 1e-3) / 1e9, 1),
+                   "speedup_over_vendor_dense": round(dense_ms / ms_per_step, 3),
+                   "note": "torch.nn.functional.conv2d (MIOpen) on the same tensors, weights dense with the zeros in"}
+
     out = {
         "metric": "effective GFLOP/s (dense-equivalent) over the layer stack; per-layer us and roofline in `layers`",
         "value": round(fl_dense / (ms_per_step * 1e-3) / 1e9, 1),
@@ -226,6 +253,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "check": check,
+        "context": context,
         "layers": table,
     }
     print(json.dumps(out))
