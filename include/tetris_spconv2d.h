@@ -118,7 +118,8 @@ int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_
 /* Measured selection, the counterpart of GetTetrisSparseConv2dTime (Tetris/spconv2d.cc:72-329): packs the filter
  * for the `max_candidates` (0 = 24) tile shapes the model of tetris_tile_select ranks best, times each on the
  * device with the real weights (1 warm-up + 3 launches on zero-filled input), times the four fastest again
- * (2 + 10 launches) and returns the fastest and its milliseconds per launch.  Allocates and frees its own device buffers; synchronises `stream`. */
+ * (2 + 10 launches) and returns the fastest and its milliseconds per launch.  Allocates and frees its own
+ * device buffers; synchronises `stream`. */
 int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int img_w, int in_channel, int out_channel,
                          int kernel_size, int stride, int padding, int max_candidates, void* stream,
                          tetris_tile* out, float* ms_out);
@@ -128,7 +129,9 @@ int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int i
  * (Tetris/spconv2d_kernel.cuh:14-21, Tetris/spconv2d_kernel.cu:163-188).  Asynchronous on `stream`.
  * d_input is NCHW [batch][in_channel][img_h][img_w], d_output NCHW [batch][out_channel][oh][ow] with
  * oh = (img_h + 2*padding - kernel_size)/stride + 1 (the reference keeps NHWC on the device; its host
- * entry points below take and return NCHW, as here).
+ * entry points below take and return NCHW, as here).  A layer with very few pixels per image is computed
+ * by several workgroups per output tile: the launch then zero-fills d_output with a kernel of its own and the
+ * workgroups add their partial sums with fp32 atomics, so the last bits can differ from run to run.
  * ---------------------------------------------------------------------------------------------- */
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
                            int stride, int padding, const tetris_tile* tile, void* stream);
