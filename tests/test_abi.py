@@ -92,3 +92,27 @@ def test_tile_select_is_sane():
         assert t.oc_per_wave * 4 * t.quads <= (64 if t.waves == 16 else 128) and t.waves in (1, 2, 4, 8, 16) and t.tile_ic >= 1
     with pytest.raises(T.TetrisError):
         T.tile_select(0, 5, 5, 3, 3, 3, 1, 1)
+
+
+def test_tile_select_answers_from_the_measured_table():
+    # shapes of the benchmark suites are answered from csrc/tuned_tiles.inc (as long as the kernel accepts the entry)
+    import re
+
+    import tetris_amd as T
+    from conftest import ROOT
+
+    rows = {}
+    with open(os.path.join(ROOT, "tetris-artifact-evalution_amd", "csrc", "tuned_tiles.inc")) as f:
+        for line in f:
+            m = re.match(r"\s*\{(\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), (\d+), \{(\d+), (\d+), (\d+), (\d+), (\d+)\}\}", line)
+            if m:
+                v = [int(x) for x in m.groups()]
+                rows.setdefault(tuple(v[:8]), tuple(v[8:]))  # the first entry of a shape wins, as in the library
+    assert len(rows) >= 100
+    hits = 0
+    for key, tile in list(rows.items())[::7]:
+        n, h, w, c, k, ks, stride, pad = key
+        t = T.tile_select(n, h, w, c, k, ks, stride, pad)
+        got = (t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic)
+        hits += got == tile
+    assert hits >= len(list(rows.items())[::7]) - 2  # an entry the current geometry checks refuse falls back to the model
