@@ -35,6 +35,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--suite", default="vgg19")
     ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--masks", metavar="NPZ", help="run the layers of a pruned network instead of --suite: a mask file "
+                    "as tests/golden/masks_*.npz (zero patterns of shipped pruned weight files, seeded values)")
+    ap.add_argument("--oc-order", choices=("balanced", "file"), default="balanced",
+                    help="output-channel order of the packs: balanced over the waves of a workgroup, or as in the filter")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
     ap.add_argument("--layer-repeat", type=int, default=30, help="timed launches per layer for the per-layer table")
@@ -77,7 +81,9 @@ def main():
         print(json.dumps({"calibrate_copy_mib": args.calibrate_copy, "dispatches": 4,
                           "bytes_read_per_dispatch": 4 * n, "bytes_written_per_dispatch": 4 * n}))
         return
-    layers = W.SUITES[args.suite]()
+    layers = W.pruned_suite(args.masks) if args.masks else W.SUITES[args.suite]()
+    if args.masks:
+        args.suite = layers[0].suite
     N = args.batch
 
     packs, tiles, xs, ys, works = [], [], [], [], []
@@ -95,7 +101,7 @@ def main():
         else:
             tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
         t0 = time.perf_counter()
-        pk = T.G950Filter.for_tile(w, tile)
+        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced" if args.oc_order == "balanced" else None)
         torch.cuda.synchronize()
         t_pack += time.perf_counter() - t0
         x = torch.from_numpy(W.make_activations(L, N)).to(dev)
@@ -184,7 +190,7 @@ def main():
     if not args.no_cpu:
         import oracle_py as O
         threads = min(O.max_threads(), 16)
-        sample_layers = W.SUITES[args.suite]()
+        sample_layers = layers
         # the same workload (every layer at the benchmark's batch) once through the oracle's packed-format conv, cut
         # short after about 25 s of wall time: a few tens of core-seconds
         budget_s, done_fl, t_cpu, used = 25.0, 0.0, 0.0, 0
@@ -250,6 +256,7 @@ def main():
         "sum_layer_us": round(t_layers * 1e6, 1) if table else None,
         "pack_ms_total": round(t_pack * 1e3, 2),
         "tile_selection": args.tile,
+        "oc_order": args.oc_order,
         "roofline": roofline,
         "cpu_baseline": cpu,
         "check": check,

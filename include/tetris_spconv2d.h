@@ -115,11 +115,22 @@ typedef struct tetris_tile {
 int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_channel, int kernel_size, int stride,
                        int padding, tetris_tile* out);
 
+/* Output-channel order for tetris_g950_create that evens out the work of the waves of a workgroup of `tile`
+ * (uses tile->oc_per_wave, waves and tile_ic).  Plays the part of SparseFilter::ReorderOutChannel
+ * (Tetris/spconv2d_utils.h:275-420) for the HIP kernel: channels sorted by their non-zero count are dealt to the
+ * workgroups' blocks of waves*oc_per_wave slots in serpentine order, then inside a block each goes to the wave
+ * where it adds least to the sum over input-channel stages of the busiest wave's entries.  On pruned networks,
+ * whose channels differ widely in density, the busiest wave of a stage holds 1.2-1.5x the mean in file order.
+ * `order_out` receives a permutation of 0..out_channel-1.  Pure host code. */
+int tetris_oc_order_balanced(const float* h_filter_oihw, int in_channel, int out_channel, int kernel_size,
+                             const tetris_tile* tile, int32_t* order_out);
+
 /* Measured selection, the counterpart of GetTetrisSparseConv2dTime (Tetris/spconv2d.cc:72-329): packs the filter
- * for the `max_candidates` (0 = 24) tile shapes the model of tetris_tile_select ranks best, times each on the
- * device with the real weights (1 warm-up + 3 launches on zero-filled input), times the four fastest again
- * (2 + 10 launches) and returns the fastest and its milliseconds per launch.  Allocates and frees its own
- * device buffers; synchronises `stream`. */
+ * for the `max_candidates` (0 = 24) tile shapes the model of tetris_tile_select ranks best (each in the
+ * output-channel order of tetris_oc_order_balanced for that tile), times each on the device with the real
+ * weights (1 warm-up + 3 launches on zero-filled input), times the four fastest again (2 + 10 launches) and
+ * returns the fastest and its milliseconds per launch.  Allocates and frees its own device buffers;
+ * synchronises `stream`. */
 int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int img_w, int in_channel, int out_channel,
                          int kernel_size, int stride, int padding, int max_candidates, void* stream,
                          tetris_tile* out, float* ms_out);

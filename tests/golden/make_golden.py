@@ -3,6 +3,9 @@
 * weights_*.npz   five shipped pruned layers, parsed by the reference's own ReadConfigAndDataFromFile
                   (tensor_utils.cc:55-82, compiled unmodified into oracle/_ref) -- data files, stored as float32
                   arrays plus the eight header ints.
+* masks_*.npz     the zero patterns of every shipped layer of two pruned networks (VGG19 at 92 %, MobileNetV1 at
+                  86 %): per layer the eight header ints and numpy.packbits(weight != 0), plus the file names.
+                  tetris_amd.workloads.pruned_suite() turns them into benchmark layers with seeded values.
 * spf_known_answers.json is NOT produced here: it is the table of FNV-1a-64 hashes and array sizes that was
   recorded from the compiled reference SparseFilter (spconv2d_utils.h) for these layers; the reference's CUDA
   headers are absent from this image so that class cannot be rebuilt here.
@@ -33,8 +36,25 @@ BIG_FILES = {
     "vgg_256": "vgg19/vgg19-92-acc-71.7/module8_0_module2_0_conv2d_3_H_56_W_56_IC_256_OC_256_KS_3_Pad_1_S_1_G_1",
 }
 
+MASK_DIRS = {"vgg19_92": "vgg19/vgg19-92-acc-71.7", "mobilenet_86": "mobilenet/mobilenet-86-acc-70.1"}
+
+
+def write_masks(tag, rel):
+    names = sorted(os.listdir(os.path.join(D, rel)))
+    arrays = {}
+    for i, fn in enumerate(names):
+        hdr, w = O.ref_read_weight_file(os.path.join(D, rel, fn))
+        arrays["hdr_%02d" % i] = np.array([hdr[k] for k in ("H", "W", "IC", "OC", "KS", "PAD", "STRIDE", "GROUPS")], np.int32)
+        arrays["bits_%02d" % i] = np.packbits((w != 0).reshape(-1))
+    out = os.path.join(HERE, "masks_%s.npz" % tag)
+    np.savez_compressed(out, names=np.array(names), source=np.array(rel), **arrays)
+    print(tag, len(names), "layers", os.path.getsize(out))
+
+
 if __name__ == "__main__":
     assert O.ref_available(), "build oracle/_ref first: make -C oracle"
+    for tag, rel in MASK_DIRS.items():
+        write_masks(tag, rel)
     for name, rel in FILES.items():
         hdr, w = O.ref_read_weight_file(os.path.join(D, rel))
         header = np.array([hdr[k] for k in ("H", "W", "IC", "OC", "KS", "PAD", "STRIDE", "GROUPS")], np.int32)

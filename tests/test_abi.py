@@ -116,3 +116,75 @@ def test_tile_select_answers_from_the_measured_table():
         got = (t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic)
         hits += got == tile
     assert hits >= len(list(rows.items())[::7]) - 2  # an entry the current geometry checks refuse falls back to the model
+
+
+def _busiest_wave_cost(w, order, g, waves, tile_ic):
+    """Sum over workgroup blocks and input-channel stages of the busiest wave's entry count (what the waves of a
+    workgroup wait for at their per-stage barrier), and the per-block sums."""
+    K, C = w.shape[:2]
+    stages = -(-C // tile_ic)
+    per = np.zeros((K, stages), np.int64)
+    for s in range(stages):
+        per[:, s] = (w[:, s * tile_ic:(s + 1) * tile_ic] != 0).reshape(K, -1).sum(1)
+    block = g * waves
+    padded = np.zeros((-(-K // block) * block, stages), np.int64)
+    padded[:K] = per[order]
+    by_block = padded.reshape(-1, waves, g, stages).sum(2).max(1).sum(1)
+    return int(by_block.sum()), by_block
+
+
+@pytest.mark.parametrize("K,C,ks,g,waves,tile_ic", [(128, 64, 3, 4, 16, 16), (255, 96, 1, 8, 8, 32), (64, 48, 3, 8, 8, 64),
+                                                   (40, 24, 3, 16, 2, 8), (7, 5, 7, 4, 4, 3)])
+def test_balanced_order_is_a_permutation_that_lowers_the_busiest_wave(K, C, ks, g, waves, tile_ic):
+    rng = np.random.default_rng(K + C)
+    # channels of very different density, some empty, as pruned networks have
+    density = np.clip(rng.lognormal(np.log(0.12), 0.8, K), 0, 0.9)
+    density[rng.random(K) < 0.1] = 0
+    w = (rng.standard_normal((K, C, ks, ks)) * (rng.random((K, C, ks, ks)) < density[:, None, None, None])).astype(np.float32)
+    tile = T.Tile(7, 2, g, waves, tile_ic)
+    order = T.oc_order_balanced(w, tile)
+    assert order.dtype == np.int32 and sorted(order.tolist()) == list(range(K))
+    ident, _ = _busiest_wave_cost(w, np.arange(K), g, waves, tile_ic)
+    bal, by_block = _busiest_wave_cost(w, order, g, waves, tile_ic)
+    assert bal <= ident
+    if K >= 4 * g * waves // 2 and K % (g * waves) == 0:
+        assert bal <= 0.92 * ident                      # a clear gain on skewed channels
+        assert by_block.max() <= 1.1 * by_block.mean()  # and no straggler workgroup
+    assert np.array_equal(order, T.oc_order_balanced(w, tile))  # deterministic
+
+
+def test_balanced_order_on_a_shipped_pruned_layer():
+    hdr, w, _ = golden_weights("vgg_64x128")  # 64 -> 128 channels, 3x3, 85 % pruned: 7 .. 165 non-zeros per channel
+    for g, waves, tile_ic in [(4, 16, 16), (8, 8, 32)]:
+        order = T.oc_order_balanced(w, T.Tile(14, 2, g, waves, tile_ic))
+        ident, _ = _busiest_wave_cost(w, np.arange(128), g, waves, tile_ic)
+        bal, _ = _busiest_wave_cost(w, order, g, waves, tile_ic)
+        assert bal <= 0.88 * ident
+
+
+def test_balanced_order_rejects_bad_arguments():
+    w = np.ones((8, 8, 1, 1), np.float32)
+    with pytest.raises(T.TetrisError):
+        T.oc_order_balanced(w, T.Tile(7, 2, 0, 8, 8))
+
+
+@pytest.mark.parametrize("masks,count", [("masks_vgg19_92.npz", 8), ("masks_mobilenet_86.npz", 13)])
+def test_pruned_suites_load_and_balance(masks, count):
+    from tetris_amd import workloads as W
+
+    layers = W.pruned_suite(os.path.join(GOLDEN, masks))
+    assert len(layers) == count
+    gains = []
+    for L in layers:
+        assert L.mask.shape == (L.K, L.C, L.ks, L.ks) and ("IC_%d_OC_%d_KS_%d" % (L.C, L.K, L.ks)) in L.name
+        assert abs((1.0 - L.sparsity) * L.mask.size - W.nnz_of(L)) < 0.5
+        if L.C < 16:
+            continue
+        w = W.make_weights(L)
+        assert np.array_equal(w != 0, L.mask)
+        tile = T.tile_select(16, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+        order = T.oc_order_balanced(w, tile)
+        ident, _ = _busiest_wave_cost(w, np.arange(L.K), tile.oc_per_wave, tile.waves, tile.tile_ic)
+        bal, _ = _busiest_wave_cost(w, order, tile.oc_per_wave, tile.waves, tile.tile_ic)
+        gains.append(bal / ident)
+    assert max(gains) <= 1.0 and np.mean(gains) <= 0.93, gains

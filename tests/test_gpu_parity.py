@@ -269,7 +269,7 @@ def test_random_shapes_with_library_tiles(env):
         w = sparse_filter(rng, K, C, ks, sp)
         x = relu_like(rng, (N, C, H, W))
         tile = T.tile_select(N, H, W, C, K, ks, stride, pad)
-        pk = T.G950Filter.for_tile(w, tile)
+        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced" if case % 2 else None)
         y = run_conv(T, torch, pk, x, K, ks, stride, pad, tile)
         ref = O.G950Pack(w, 32, 8).conv(x, stride, pad, threads=min(16, O.max_threads()))
         err = max_rel_err(y, ref)
@@ -277,3 +277,27 @@ def test_random_shapes_with_library_tiles(env):
         variants.add((tile.waves, tile.quads))
         pk.close()
     assert len(variants) >= 3, variants
+
+
+@pytest.mark.parametrize("masks", ["masks_vgg19_92.npz", "masks_mobilenet_86.npz"])
+def test_pruned_networks_in_balanced_channel_order(env, masks):
+    # The zero patterns of two shipped pruned networks (channels of very different density, some empty), every
+    # layer at full resolution and batch 2, packed in the output-channel order that balances the waves.
+    T, torch, O = env
+    from conftest import GOLDEN
+    from tetris_amd import workloads as W
+
+    layers = W.pruned_suite(os.path.join(GOLDEN, masks))
+    assert len(layers) >= 8
+    for L in layers:
+        w, x = W.make_weights(L), W.make_activations(L, 2)
+        assert int((w != 0).sum()) == W.nnz_of(L)
+        tile = T.tile_select(2, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+        order = T.oc_order_balanced(w, tile)
+        pk = T.G950Filter.for_tile(w, tile, oc_order=order)
+        assert np.array_equal(pk.host_arrays()["oc_order"][:L.K], order)
+        y = run_conv(T, torch, pk, x, L.K, L.ks, L.stride, L.pad, tile)
+        ref = O.G950Pack(w, 32, 8).conv(x, L.stride, L.pad, threads=min(16, O.max_threads()))
+        err = max_rel_err(y, ref)
+        assert err <= TOL, (L.name, tile, err)
+        pk.close()

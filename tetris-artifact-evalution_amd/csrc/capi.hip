@@ -116,16 +116,16 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
   tetris_tile tile{};
   int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &tile);
   if (rc) return rc;
-  // The spf entry point of the reference fixes TILE_IC = 128 and never regroups differently per tile;
-  // here it fixes the packer arguments the same way and leaves the kernel tile to the selector.
-  const int ref_tile_ic = fixed_spf_config ? 128 : 32;
-  tetris_spf* spf = nullptr;
+  // apply_reorder: the reference regroups output channels for its warps (ReorderOutChannel); the kernel here
+  // gets the order that balances its own waves instead.  The results do not depend on the order.
+  // The reference's spf entry point fixes its tile template arguments; here both entry points leave the
+  // tile to the selector.
+  (void)fixed_spf_config;
   std::vector<int32_t> order;
   if (apply_reorder) {
-    // keep the reference's output-channel regrouping for the slot order of the kernel's pack
-    rc = tetris_spf_create(h_filter, C, K, ks, ref_tile_ic, 1, 1, TETRIS_REORDER_OUT_CHANNEL, &spf);
+    order.resize(K);
+    rc = balance_oc_order(h_filter, C, K, ks, tile, order.data());
     if (rc) return rc;
-    order = spf->oc_permutation;
   }
   tetris_g950* pack = nullptr;
   rc = tetris_g950_create(h_filter, C, K, ks, tile.tile_ic, tile.oc_per_wave, apply_reorder ? order.data() : nullptr,
@@ -136,7 +136,6 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
     if (d_in) (void)hipFree(d_in);
     if (d_out) (void)hipFree(d_out);
     tetris_g950_destroy(pack);
-    tetris_spf_destroy(spf);
     return code;
   };
   if (rc) return done(rc);
@@ -193,15 +192,17 @@ static int spf_ensure_device(tetris_spf* f) {
   return TETRIS_OK;
 }
 
-// The kernel's own pack of this filter for `tile_ic` staged input channels, in the same slot order.
-static int spf_kernel_pack(tetris_spf* f, int tile_ic, int oc_per_wave, hipStream_t stream, tetris_g950** out) {
+// The kernel's own pack of this filter for tile `t`, with the output-channel order that balances the tile's waves.
+static int spf_kernel_pack(tetris_spf* f, const tetris_tile& t, hipStream_t stream, tetris_g950** out) {
   std::lock_guard<std::mutex> lock(f->mu);
-  const std::pair<int, int> key(tile_ic, oc_per_wave);
+  const std::array<int, 3> key{t.tile_ic, t.oc_per_wave, t.waves};
   auto it = f->kernel_packs.find(key);
   if (it == f->kernel_packs.end()) {
+    std::vector<int32_t> order(f->K);
+    int rc = balance_oc_order(f->filter.data(), f->C, f->K, f->ks, t, order.data());
+    if (rc) return rc;
     tetris_g950* p = nullptr;
-    int rc = tetris_g950_create(f->filter.data(), f->C, f->K, f->ks, tile_ic, oc_per_wave, f->oc_permutation.data(),
-                                stream, &p);
+    rc = tetris_g950_create(f->filter.data(), f->C, f->K, f->ks, t.tile_ic, t.oc_per_wave, order.data(), stream, &p);
     if (rc) return rc;
     it = f->kernel_packs.emplace(key, p).first;
   }
@@ -269,6 +270,12 @@ int tetris_tile_select(int N, int H, int W, int C, int K, int ks, int stride, in
   return choose_tile(N, H, W, C, K, ks, stride, pad, out);
 }
 
+int tetris_oc_order_balanced(const float* h_filter, int C, int K, int ks, const tetris_tile* tile, int32_t* order_out) {
+  if (!h_filter || !tile || !order_out) return fail(TETRIS_EINVAL, "null argument");
+  if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs) return fail(TETRIS_EINVAL, "bad filter shape");
+  return balance_oc_order(h_filter, C, K, ks, *tile, order_out);
+}
+
 int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int K, int ks, int stride, int pad,
                          int max_candidates, void* stream_, tetris_tile* out, float* ms_out) {
   if (!h_filter || !out) return fail(TETRIS_EINVAL, "null argument");
@@ -281,7 +288,8 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
   const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
   const size_t f_bytes = sizeof(float) * (size_t)C * K * ks * ks;
   float *d_in = nullptr, *d_out = nullptr, *d_f = nullptr;
-  std::map<std::pair<int, int>, tetris_g950*> packs;
+  std::map<std::array<int, 3>, tetris_g950*> packs;  // by (tile_ic, oc_per_wave, waves): what the pack and its order depend on
+  std::vector<int32_t> order(K);
   auto done = [&](int code) {
     for (auto& kv : packs) tetris_g950_destroy(kv.second);
     if (d_in) (void)hipFree(d_in);
@@ -305,11 +313,12 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
   std::vector<std::pair<float, tetris_tile>> timed;
   for (const tetris_tile& t : ranked) {
     if ((int)timed.size() >= max_candidates) break;
-    const std::pair<int, int> key(t.tile_ic, t.oc_per_wave);
+    const std::array<int, 3> key{t.tile_ic, t.oc_per_wave, t.waves};
     auto it = packs.find(key);
     if (it == packs.end()) {
       tetris_g950* p = nullptr;
-      rc = tetris_g950_create_device(d_f, C, K, ks, t.tile_ic, t.oc_per_wave, nullptr, stream, &p);
+      rc = balance_oc_order(h_filter, C, K, ks, t, order.data());
+      if (rc == TETRIS_OK) rc = tetris_g950_create_device(d_f, C, K, ks, t.tile_ic, t.oc_per_wave, order.data(), stream, &p);
       if (rc) return done(rc);
       it = packs.emplace(key, p).first;
     }
@@ -327,8 +336,8 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
   for (size_t i = 0; i < timed.size() && i < 4; ++i) {
     const tetris_tile& t = timed[i].second;
     float ms = 0;
-    rc = time_launches(packs[std::make_pair(t.tile_ic, t.oc_per_wave)], d_in, d_out, N, H, W, stride, pad, &t, stream, 2,
-                       10, &ms);
+    rc = time_launches(packs[{t.tile_ic, t.oc_per_wave, t.waves}], d_in, d_out, N, H, W, stride, pad, &t, stream, 2, 10,
+                       &ms);
     if (rc) return done(rc);
     if (ms < best_ms) {
       best_ms = ms;
@@ -363,7 +372,7 @@ int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, cons
   int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &t);
   if (rc) return rc;
   tetris_g950* pack = nullptr;
-  rc = spf_kernel_pack(f, t.tile_ic, t.oc_per_wave, static_cast<hipStream_t>(stream), &pack);
+  rc = spf_kernel_pack(f, t, static_cast<hipStream_t>(stream), &pack);
   if (rc) return rc;
   return run_launch(pack, d_in, d_out, N, H, W, stride, pad, &t, static_cast<hipStream_t>(stream));
 }

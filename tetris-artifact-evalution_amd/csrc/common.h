@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <array>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -154,7 +155,7 @@ struct tetris_spf {
   int32_t *d_offsets = nullptr, *d_stage_len = nullptr, *d_position = nullptr, *d_oc_permutation = nullptr;
   float* d_values = nullptr;
   std::vector<float> filter;                              // dense copy the kernel's packs are made from
-  std::map<std::pair<int, int>, tetris_g950*> kernel_packs;  // by (staged input channels, slots per wave)
+  std::map<std::array<int, 3>, tetris_g950*> kernel_packs;  // by (staged input channels, slots per wave, waves)
   std::mutex mu;
 };
 
@@ -172,6 +173,9 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
 int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t);
 // every tile shape the kernel can run for the layer, cheapest first by the selector's time model
 int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked);
+
+// output-channel order (a permutation of 0..K-1) that balances the waves of a workgroup for tile `t`
+int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_tile& t, int32_t* order);
 
 // spconv2d_kernel.hip
 // launches the conv (after a zero fill of the output when the geometry splits the channel reduction)

@@ -311,4 +311,79 @@ int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, 
   return TETRIS_OK;
 }
 
+// Output-channel order that evens out the work inside a workgroup.  A wave walks the entries of its
+// `oc_per_wave` slots stage by stage and the waves of a workgroup meet at a barrier after every stage, so a
+// stage costs the workgroup what its busiest wave holds.  Pruned networks have output channels of very
+// different density (some are empty): in file order the busiest wave of a stage carries 1.2-1.5x the mean.
+// The channels are sorted by their number of non-zeros and dealt to the workgroups' blocks of
+// waves*oc_per_wave slots in serpentine order (blocks of equal total work: no straggler workgroup); inside a
+// block each channel, heaviest first, goes to the wave where it raises the sum over stages of the busiest
+// wave's count the least.  Plays the part of ReorderOutChannel (Tetris/spconv2d_utils.h:275-420), whose
+// own objective -- lanes of a warp with alike channels -- does not fit a wave that sums its channels.
+int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_tile& t, int32_t* order) {
+  const int G = t.oc_per_wave, waves = t.waves, tile_ic = t.tile_ic;
+  if (G <= 0 || waves <= 0 || tile_ic <= 0) return fail(TETRIS_EINVAL, "bad tile");
+  const int S = ceil_div(C, tile_ic), B = G * waves, nblocks = ceil_div(K, B), taps = ks * ks;
+  std::vector<int32_t> per((size_t)K * S, 0);
+  std::vector<int64_t> total(K, 0);
+  for (int k = 0; k < K; ++k)
+    for (int c = 0; c < C; ++c) {
+      const float* w = filter + ((size_t)k * C + c) * taps;
+      int n = 0;
+      for (int i = 0; i < taps; ++i) n += w[i] != 0.f;
+      per[(size_t)k * S + c / tile_ic] += n;
+      total[k] += n;
+    }
+  std::vector<int32_t> sorted(K);
+  for (int k = 0; k < K; ++k) sorted[k] = k;
+  std::stable_sort(sorted.begin(), sorted.end(), [&](int32_t a, int32_t b) { return total[a] > total[b]; });
+  // serpentine deal; the last block may hold fewer than B channels
+  std::vector<std::vector<int32_t>> blocks(nblocks);
+  {
+    int b = 0, d = 1;
+    for (int32_t k : sorted) {
+      while ((int)blocks[b].size() >= std::min(B, K - b * B)) {
+        b += d;
+        if (b < 0 || b >= nblocks) { d = -d; b += d; }
+      }
+      blocks[b].push_back(k);
+      b += d;
+      if (b < 0 || b >= nblocks) { d = -d; b += d; }
+    }
+  }
+  std::vector<int64_t> load((size_t)waves * S), busiest(S);
+  std::vector<std::vector<int32_t>> members(waves);
+  int32_t* o = order;
+  for (const std::vector<int32_t>& blk : blocks) {
+    std::fill(load.begin(), load.end(), 0);
+    std::fill(busiest.begin(), busiest.end(), 0);
+    for (auto& m : members) m.clear();
+    const int len = (int)blk.size();
+    for (int32_t k : blk) {
+      int best = -1;
+      int64_t best_cost = 0, best_sum = 0;
+      for (int w = 0; w < waves; ++w) {
+        const int cap = std::min(G, std::max(0, len - w * G));  // slots of this wave that hold a channel
+        if ((int)members[w].size() >= cap) continue;
+        int64_t cost = 0, sum = 0;
+        for (int s = 0; s < S; ++s) {
+          cost += std::max(busiest[s], load[(size_t)w * S + s] + per[(size_t)k * S + s]);
+          sum += load[(size_t)w * S + s];
+        }
+        if (best < 0 || cost < best_cost || (cost == best_cost && sum < best_sum)) {
+          best = w; best_cost = cost; best_sum = sum;
+        }
+      }
+      for (int s = 0; s < S; ++s) {
+        load[(size_t)best * S + s] += per[(size_t)k * S + s];
+        busiest[s] = std::max(busiest[s], load[(size_t)best * S + s]);
+      }
+      members[best].push_back(k);
+    }
+    for (int w = 0; w < waves; ++w)
+      for (int32_t k : members[w]) *o++ = k;
+  }
+  return TETRIS_OK;
+}
+
 }  // namespace tetris

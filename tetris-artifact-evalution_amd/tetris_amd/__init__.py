@@ -97,6 +97,8 @@ _lib.tetris_g950_destroy.argtypes = [C.c_void_p]
 _lib.tetris_g950_destroy.restype = None
 _lib.tetris_g950_host_arrays.argtypes = [C.c_void_p, C.POINTER(_G950Arrays)]
 _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
+_lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(Tile),
+                                          np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")]
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
 _lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile),
                                                                                                 C.c_void_p]
@@ -200,6 +202,11 @@ class G950Filter:
 
     @classmethod
     def for_tile(cls, filter, tile, oc_order=None, stream=0):
+        """oc_order: None (file order), an int32 permutation, or "balanced" (oc_order_balanced for this tile)."""
+        if isinstance(oc_order, str):
+            if oc_order != "balanced":
+                raise ValueError("oc_order: None, a permutation or 'balanced'")
+            oc_order = oc_order_balanced(filter, tile)
         return cls(filter, tile.tile_ic, tile.oc_per_wave, oc_order, stream)
 
     def __init__(self, filter, tile_ic, oc_per_wave, oc_order=None, stream=0, device_ptr=None, shape=None):
@@ -255,6 +262,15 @@ def tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, strid
     _check(_lib.tetris_tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
                                    C.byref(t)))
     return t
+
+
+def oc_order_balanced(filter, tile):
+    """Output-channel order that evens out the waves of a workgroup of `tile` (tetris_oc_order_balanced)."""
+    w = np.ascontiguousarray(filter, np.float32)
+    K, Cc, ks, _ = w.shape
+    order = np.empty(K, np.int32)
+    _check(_lib.tetris_oc_order_balanced(w, Cc, K, ks, C.byref(tile), order))
+    return order
 
 
 def tile_autotune(filter, batch, img_h, img_w, stride, padding, max_candidates=0, stream=0):

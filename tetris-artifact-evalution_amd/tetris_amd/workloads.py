@@ -8,13 +8,17 @@ into floats with explicit integer arithmetic (no library distribution objects).
   activations  NCHW fp32, uniform [0, 1) with each element zeroed with probability 1/2 (ReLU-like)
 The reference draws its inputs from rand() seeded with time(0) (Tetris/spconv2d.cc:377,
 Tetris/tensor_utils.cc:9-14), which cannot be reproduced, and reads pruned weights from text files.
+
+pruned_suite() makes layers whose zero pattern is that of such a pruned network (a file of bit-packed masks), with
+seeded values: the time of a launch depends on where the non-zeros are, not on what they are.
 """
+import os
 import zlib
 from collections import namedtuple
 
 import numpy as np
 
-Layer = namedtuple("Layer", "suite index name C H W K ks stride pad sparsity")
+Layer = namedtuple("Layer", "suite index name C H W K ks stride pad sparsity mask", defaults=(None,))
 
 _M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
 BASE_SEED = 0x7E7A15
@@ -44,6 +48,8 @@ def make_weights(layer, base_seed=BASE_SEED):
     u2 = _uniform01(_splitmix64(seed ^ 0xA5A5A5A5, n))
     w = (0.05 * np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2)).astype(np.float32)
     w[w == 0] = np.float32(1e-6)  # keep the non-zero count exact
+    if layer.mask is not None:
+        return np.where(layer.mask, w.reshape(layer.mask.shape), np.float32(0))
     nzero = int(round(layer.sparsity * n))
     keys = _splitmix64(seed ^ 0x3C3C3C3C, n)
     w[np.argsort(keys, kind="stable")[:nzero]] = 0.0
@@ -66,6 +72,8 @@ def out_hw(layer):
 
 
 def nnz_of(layer):
+    if layer.mask is not None:
+        return int(layer.mask.sum())
     n = layer.K * layer.C * layer.ks * layer.ks
     return n - int(round(layer.sparsity * n))
 
@@ -166,6 +174,21 @@ def yolov3():
     head("head26", 768, 256, 26)
     add("route26", 256, 26, 128, 1, 1)
     head("head52", 384, 128, 52)
+    return out
+
+
+def pruned_suite(npz_path):
+    """The layers of a pruned network as recorded in a mask file: `names` (the weight files' names), and per layer
+    i `hdr_%02d` (the eight header ints H W IC OC KS PAD STRIDE GROUPS of Tetris/tensor_utils.cc:66) and `bits_%02d`
+    (numpy.packbits of `weight != 0` in OIHW order)."""
+    z = np.load(npz_path)
+    suite = os.path.splitext(os.path.basename(npz_path))[0]
+    out = []
+    for i, name in enumerate(z["names"]):
+        H, Wd, C, K, ks, pad, stride, _ = (int(v) for v in z["hdr_%02d" % i])
+        n = K * C * ks * ks
+        mask = np.unpackbits(z["bits_%02d" % i])[:n].reshape(K, C, ks, ks).astype(bool)
+        out.append(Layer(suite, i, str(name), C, H, Wd, K, ks, stride, pad, 1.0 - float(mask.sum()) / n, mask))
     return out
 
 
