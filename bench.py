@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--dense-baseline", action="store_true",
                     help="also time the vendor's dense fp32 convolution (MIOpen through torch) on the same layers, as "
                          "context (the reference compares with cuDNN the same way, Tetris/cuda_utils.cc:6-132)")
+    ap.add_argument("--csr-baseline", action="store_true",
+                    help="also time the vendor sparse-library path on the same tensors: im2col (torch unfold) + CSR x "
+                    "dense product (torch.sparse.mm, rocSPARSE), the counterpart of the reference's cusparse_test")
     ap.add_argument("--calibrate-copy", type=int, metavar="MIB", default=0,
                     help="instead of the benchmark, run one elementwise copy kernel over MIB MiB (reads MIB, writes MIB): "
                          "the known-size dispatch that scales the FETCH_SIZE / WRITE_SIZE counters")
@@ -242,6 +245,32 @@ def main():
                    "vendor_dense_fp32_gflops": round(fl_dense / (dense_ms * 1e-3) / 1e9, 1),
                    "speedup_over_vendor_dense": round(dense_ms / ms_per_step, 3),
                    "note": "torch.nn.functional.conv2d (MIOpen) on the same tensors, weights dense with the zeros in"}
+
+    if args.csr_baseline:
+        import torch.nn.functional as F
+        context = context or {}
+        try:
+            csr = [torch.from_numpy(W.make_weights(L).reshape(L.K, -1)).to(dev).to_sparse_csr() for L in layers]
+
+            def csr_step():
+                for L, x, a in zip(layers, xs, csr):
+                    for n in range(N):  # one image at a time keeps the unfolded matrix small (C*ks*ks x OH*OW)
+                        torch.sparse.mm(a, F.unfold(x[n:n + 1], L.ks, padding=L.pad, stride=L.stride)[0])
+
+            csr_step()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            csr_step()
+            e1.record()
+            torch.cuda.synchronize()
+            csr_ms = e0.elapsed_time(e1)
+            context.update({"vendor_csr_im2col_ms_per_step": round(csr_ms, 3),
+                            "speedup_over_vendor_csr": round(csr_ms / ms_per_step, 2),
+                            "csr_note": "per image: torch unfold (im2col) + torch.sparse.mm (CSR weights x dense "
+                                        "columns, rocSPARSE); one pass, outputs discarded"})
+        except Exception as e:  # the sparse library path is context, not the product
+            context.update({"vendor_csr_im2col_ms_per_step": None, "csr_note": "failed: %r" % (e,)})
 
     out = {
         "metric": "effective GFLOP/s (dense-equivalent) over the layer stack; per-layer us and roofline in `layers`",
