@@ -72,3 +72,59 @@ def test_cli_missing_file_behaves_like_the_reference():
     p = subprocess.run([os.path.join(BIN, "spconv2d_test"), "/nonexistent/layer", "1"], capture_output=True, text=True,
                        timeout=60)
     assert p.returncode == 1 and "Open file error." in p.stdout  # Tetris/tensor_utils.cc:61-64
+
+
+CANNED = """args : 3 ./spconv2d_test.o layer 4
+
+GPU Device 0: "AMD Instinct MI355X" (gfx950, 256 compute units)
+
+[Config] sparsity = 0.899902, nnz = 7380, batch_size = 4, img_h = 56, img_w = 56, in_channel = 64, out_channel = 128, kernel_size = 3, padding = 1, stride = 1
+Time of Spconv2d :0.012345ms
+FLOPS of Spconv2d :136.5T
+"""
+
+
+def test_timing_driver_parses_and_writes_the_reference_csv(tmp_path):
+    # host logic of the per-folder timing loop (counterpart of evalution/conv2d_timing.py), with a stand-in binary
+    from tetris_amd import timing
+
+    cfg, ms, tf = timing.parse_output(CANNED)
+    assert (ms, tf) == (0.012345, 136.5) and cfg["kernel_size"] == "3" and cfg["nnz"] == "7380" and cfg["stride"] == "1"
+    assert timing.parse_output("nothing useful\n") == ({}, -1.0, -1.0)
+    folder = tmp_path / "net-90-acc-1.0"
+    folder.mkdir()
+    rng = np.random.default_rng(0)
+    for i in range(3):
+        w = sparse_filter(rng, 8, 4, 3, 0.5)
+        timing.write_weight_file(str(folder / ("conv_%d" % i)), w, 9, 9, 1, 1)
+    import tetris_amd as T
+    hdr, w2 = T.ReadConfigAndDataFromFile(str(folder / "conv_2"))[:2]
+    assert np.array_equal(w2.reshape(w.shape), w)  # nine significant digits round-trip fp32
+    fake = tmp_path / "fake_bin"
+    fake.write_text("#!/bin/sh\ncat <<'EOT'\n" + CANNED + "EOT\n")
+    fake.chmod(0o755)
+    csv, rows = timing.time_folder(str(fake), str(folder), 4, str(tmp_path / "logs"))
+    assert os.path.basename(csv) == "net-90-acc-1.0_batch_4.csv"
+    assert open(csv).read().splitlines() == [",op_name,spconv2d"] + ["%d,conv_%d,%.5f" % (i, i, 0.012345) for i in range(3)]
+    log = open(str(tmp_path / "logs" / "net-90-acc-1.0_batch_4.log")).read()
+    assert log.count("# Run[") == 3 and "spconv2d: time = 0.0123" in log
+    bad = tmp_path / "bad_bin"
+    bad.write_text("#!/bin/sh\nexit 3\n")
+    bad.chmod(0o755)
+    with pytest.raises(RuntimeError):
+        timing.time_layer(str(bad), str(folder / "conv_0"), 1)
+
+
+@pytest.mark.gpu
+def test_timing_driver_on_the_real_binary(tmp_path):
+    from tetris_amd import timing
+    from tetris_amd import workloads as W
+
+    layers = [W.Layer("tiny", i, "l%d" % i, c, hw, hw, k, ks, st, ks // 2, 0.8)
+              for i, (c, hw, k, ks, st) in enumerate([(16, 14, 32, 3, 1), (24, 10, 20, 1, 1), (8, 21, 16, 3, 2)])]
+    folder = str(tmp_path / "tiny-80")
+    assert timing.write_layers(layers, folder) == 3
+    csv, rows = timing.time_folder(os.path.join(BIN, "spconv2d_test"), folder, 2, str(tmp_path / "logs"))
+    assert len(rows) == 3 and all(0 < ms < 50 for _, ms in rows)
+    lines = open(csv).read().splitlines()
+    assert lines[0] == ",op_name,spconv2d" and len(lines) == 4 and lines[1].startswith("0,000_l0_H_14_W_14_IC_16_OC_32_KS_3")

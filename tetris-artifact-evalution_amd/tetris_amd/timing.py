@@ -1,0 +1,115 @@
+"""Per-layer timing over a folder of weight files: the counterpart of the reference's evalution/conv2d_timing.py
+(its Tetris column) on this library's command-line driver.
+
+    python -m tetris_amd.timing --weights DIR [--batch 1 4 8 16] [--log-dir DIR] [--bin PATH]
+    python -m tetris_amd.timing --write-suite vgg19 DIR        # the synthetic suite as weight files
+    python -m tetris_amd.timing --write-masks MASKS.npz DIR    # a pruned network's layers (seeded values)
+
+For every weight file (the reference's text format: eight header ints `H W IC OC KS PAD STRIDE GROUPS`, then the
+OIHW values, Tetris/tensor_utils.cc:55-82) and batch size it starts `bin/spconv2d_test <file> <batch>` as a child
+process and reads the lines the reference's harness reads (conv2d_timing.py:51-79): `[Config] k = v, ...`,
+`Time of Spconv2d :<ms>ms`, `FLOPS of Spconv2d :<x>T`.  Per batch size it writes, like the reference
+(conv2d_timing.py:101-198), `<folder>_batch_<N>.csv` (columns: row index, op_name, spconv2d in ms with five decimals)
+and `<folder>_batch_<N>.log`.  Only the Tetris column exists here: the vendor baselines of the reference are not part
+of this library.
+"""
+import argparse
+import os
+import subprocess
+import sys
+
+VENDOR = "spconv2d"
+
+
+def parse_output(text):
+    """-> (config dict, milliseconds, TFLOPS) from the driver's stdout; -1.0 where a line is missing."""
+    config, ms, tflops = {}, -1.0, -1.0
+    for line in text.splitlines():
+        line = line.strip()
+        if "FLOPS of" in line:
+            tflops = float(line.split(" :")[1][:-1])
+        if "Time of" in line:
+            ms = float(line.split(" :")[1][:-2])
+        if "[Config]" in line:
+            for item in line.split("[Config] ")[1].split(", "):
+                k, v = item.split(" = ")
+                config[k] = v
+    return config, ms, tflops
+
+
+def time_layer(binary, weight_file, batch, timeout=600):
+    p = subprocess.run([binary, weight_file, str(batch)], capture_output=True, text=True, timeout=timeout)
+    if p.returncode != 0:
+        raise RuntimeError("%s %s %d: exit %d\n%s%s" % (binary, weight_file, batch, p.returncode, p.stdout[-2000:],
+                                                      p.stderr[-2000:]))
+    return parse_output(p.stdout)
+
+
+def time_folder(binary, folder, batch, log_dir):
+    folder = folder.rstrip("/")
+    tag = "%s_batch_%d" % (os.path.basename(folder), batch)
+    os.makedirs(log_dir, exist_ok=True)
+    rows = []
+    with open(os.path.join(log_dir, tag + ".log"), "w") as log:
+        for idx, op in enumerate(sorted(os.listdir(folder))):
+            path = os.path.join(folder, op)
+            if not os.path.isfile(path):
+                continue
+            log.write("# Run[%d]: %s\n" % (idx, path))
+            config, ms, tflops = time_layer(binary, path, batch)
+            log.write("%r\n%s: time = %.5fms, FLOPS = %.5fT\n%s\n\n" % (config, VENDOR, ms, tflops, "-" * 84))
+            log.flush()
+            rows.append((op, ms))
+    csv = os.path.join(log_dir, tag + ".csv")
+    with open(csv, "w") as f:
+        f.write(",op_name,%s\n" % VENDOR)
+        for i, (op, ms) in enumerate(rows):
+            f.write("%d,%s,%.5f\n" % (i, op, ms))
+    return csv, rows
+
+
+def write_weight_file(path, w, H, W, pad, stride, groups=1):
+    K, C, ks, _ = w.shape
+    with open(path, "w") as f:
+        f.write("%d %d %d %d %d %d %d %d\n" % (H, W, C, K, ks, pad, stride, groups))
+        f.write(" ".join("%.9g" % v for v in w.reshape(-1).tolist()))
+        f.write("\n")
+
+
+def write_layers(layers, out_dir):
+    from tetris_amd import workloads as W
+    os.makedirs(out_dir, exist_ok=True)
+    for L in layers:
+        name = "%03d_%s_H_%d_W_%d_IC_%d_OC_%d_KS_%d_Pad_%d_S_%d_G_1" % (L.index, L.name.split("_H_")[0], L.H, L.W, L.C,
+                                                                        L.K, L.ks, L.pad, L.stride)
+        write_weight_file(os.path.join(out_dir, name), W.make_weights(L), L.H, L.W, L.pad, L.stride)
+    return len(layers)
+
+
+def main(argv=None):
+    here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--weights", metavar="DIR", help="folder of weight files to time")
+    ap.add_argument("--batch", nargs="+", type=int, default=[1])
+    ap.add_argument("--log-dir", default="timing_out")
+    ap.add_argument("--bin", default=os.path.join(here, "bin", "spconv2d_test"))
+    ap.add_argument("--write-suite", nargs=2, metavar=("SUITE", "DIR"))
+    ap.add_argument("--write-masks", nargs=2, metavar=("NPZ", "DIR"))
+    args = ap.parse_args(argv)
+    if args.write_suite or args.write_masks:
+        from tetris_amd import workloads as W
+        layers = W.SUITES[args.write_suite[0]]() if args.write_suite else W.pruned_suite(args.write_masks[0])
+        out_dir = (args.write_suite or args.write_masks)[1]
+        print("wrote %d weight files to %s" % (write_layers(layers, out_dir), out_dir))
+    if args.weights:
+        if not os.path.isfile(args.bin):
+            sys.exit("timing: %s is not built (make -C %s)" % (args.bin, here))
+        for n in args.batch:
+            csv, rows = time_folder(args.bin, args.weights, n, args.log_dir)
+            print("batch %d: %d layers, %.3f ms in total -> %s" % (n, len(rows), sum(ms for _, ms in rows), csv), flush=True)
+    elif not (args.write_suite or args.write_masks):
+        ap.error("nothing to do: give --weights, --write-suite or --write-masks")
+
+
+if __name__ == "__main__":
+    main()
