@@ -115,6 +115,15 @@ typedef struct tetris_tile {
 int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_channel, int kernel_size, int stride,
                        int padding, tetris_tile* out);
 
+/* Persisted tile selection: reads rows `{N, H, W, C, K, ks, stride, pad, {lanes_w, quads, oc_per_wave, waves,
+ * tile_ic}},` (the format of csrc/tuned_tiles.inc, which `python -m tetris_amd.tune --out FILE` writes from
+ * tetris_tile_autotune runs; other lines are skipped) and makes tetris_tile_select, and every entry point that
+ * chooses the tile itself, answer from them before the built-in table.  Plays the part of the reference's static
+ * per-layer cache of the exhaustive search (Tetris/spconv2d.cc:90, 285-329), kept across processes.  A row whose
+ * tile the kernel's checks refuse is ignored at look-up.  *rows_out (may be NULL) receives the rows read.
+ * Process-wide; may be called several times (later files win). */
+int tetris_tile_table_load(const char* path, int* rows_out);
+
 /* Output-channel order for tetris_g950_create that evens out the work of the waves of a workgroup of `tile`
  * (uses tile->oc_per_wave, waves and tile_ic).  Plays the part of SparseFilter::ReorderOutChannel
  * (Tetris/spconv2d_utils.h:275-420) for the HIP kernel: channels sorted by their non-zero count are dealt to the

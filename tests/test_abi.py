@@ -188,3 +188,23 @@ def test_pruned_suites_load_and_balance(masks, count):
         bal, _ = _busiest_wave_cost(w, order, tile.oc_per_wave, tile.waves, tile.tile_ic)
         gains.append(bal / ident)
     assert max(gains) <= 1.0 and np.mean(gains) <= 0.93, gains
+
+
+def test_tile_table_loaded_at_run_time_wins_over_the_built_in_one(tmp_path):
+    shape = (3, 37, 41, 24, 40, 3, 1, 1)  # in no built-in table
+    model = T.tile_select(*shape)
+    want = (5, 1, 8, 2, 8)
+    assert (model.lanes_w, model.quads, model.oc_per_wave, model.waves, model.tile_ic) != want
+    table = tmp_path / "tiles.inc"
+    table.write_text("// Generated elsewhere\n"
+                     "    {3, 37, 41, 24, 40, 3, 1, 1, {5, 1, 8, 2, 8}},  // mine: 12.3 us\n"
+                     "    {3, 38, 41, 24, 40, 3, 1, 1, {62, 4, 32, 16, 4096}},  // a tile the kernel refuses\n"
+                     "not a row\n")
+    assert T.tile_table_load(str(table)) == 2
+    t = T.tile_select(*shape)
+    assert (t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic) == want
+    bad = T.tile_select(3, 38, 41, 24, 40, 3, 1, 1)  # refused row: falls through to the model
+    assert (bad.lanes_w, bad.quads, bad.oc_per_wave, bad.waves, bad.tile_ic) != (62, 4, 32, 16, 4096)
+    with pytest.raises(T.TetrisError) as e:
+        T.tile_table_load(str(tmp_path / "missing"))
+    assert e.value.code == T.EIO

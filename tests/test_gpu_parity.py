@@ -301,3 +301,18 @@ def test_pruned_networks_in_balanced_channel_order(env, masks):
         err = max_rel_err(y, ref)
         assert err <= TOL, (L.name, tile, err)
         pk.close()
+
+
+def test_tile_from_a_table_loaded_at_run_time(env, tmp_path):
+    T, torch, O = env
+    N, C, H, W, K, ks = 3, 24, 37, 41, 40, 3
+    table = tmp_path / "tiles.inc"
+    table.write_text("    {3, 37, 41, 24, 40, 3, 1, 1, {5, 1, 8, 2, 8}},\n")
+    assert T.tile_table_load(str(table)) == 1
+    tile = T.tile_select(N, H, W, C, K, ks, 1, 1)
+    assert (tile.lanes_w, tile.quads, tile.oc_per_wave, tile.waves, tile.tile_ic) == (5, 1, 8, 2, 8)
+    rng = np.random.default_rng(5)
+    w, x = sparse_filter(rng, K, C, ks, 0.85), relu_like(rng, (N, C, H, W))
+    pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+    y = run_conv(T, torch, pk, x, K, ks, 1, 1, None)  # NULL tile: the library chooses, from the loaded row
+    assert max_rel_err(y, O.host_conv2d(x, w, 1, 1, threads=4)) <= TOL

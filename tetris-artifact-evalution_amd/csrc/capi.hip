@@ -270,6 +270,11 @@ int tetris_tile_select(int N, int H, int W, int C, int K, int ks, int stride, in
   return choose_tile(N, H, W, C, K, ks, stride, pad, out);
 }
 
+int tetris_tile_table_load(const char* path, int* rows_out) {
+  if (!path) return fail(TETRIS_EINVAL, "null argument");
+  return load_tile_table(path, rows_out);
+}
+
 int tetris_oc_order_balanced(const float* h_filter, int C, int K, int ks, const tetris_tile* tile, int32_t* order_out) {
   if (!h_filter || !tile || !order_out) return fail(TETRIS_EINVAL, "null argument");
   if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs) return fail(TETRIS_EINVAL, "bad filter shape");

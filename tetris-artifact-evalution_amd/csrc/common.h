@@ -171,6 +171,8 @@ int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** en
 // tile_select.cpp
 int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile& t, Geom* g);
 int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t);
+// reads rows in the format of tuned_tiles.inc; choose_tile looks them up before the built-in table
+int load_tile_table(const char* path, int* rows_out);
 // every tile shape the kernel can run for the layer, cheapest first by the selector's time model
 int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked);
 

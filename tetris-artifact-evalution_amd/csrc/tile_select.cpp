@@ -6,6 +6,8 @@
 #include <algorithm>
 #include <climits>
 #include <cmath>
+#include <cstdio>
+#include <mutex>
 #include <utility>
 
 #include "common.h"
@@ -287,18 +289,58 @@ struct Tuned {
 const Tuned kTuned[] = {
 #include "tuned_tiles.inc"
     {0, 0, 0, 0, 0, 0, 0, 0, {0, 0, 0, 0, 0}}};
+
+// Rows a caller loaded at run time (tetris_tile_table_load); they are looked up before the built-in ones.
+std::mutex g_loaded_mu;
+std::vector<Tuned> g_loaded;
+
+// trust a table row only as far as the kernel's own checks go
+bool usable(const Tuned& e) {
+  tetris_g950 shape;
+  shape.C = e.C; shape.K = e.K; shape.ks = e.ks; shape.tile_ic = e.tile.tile_ic; shape.g = e.tile.oc_per_wave;
+  if (e.tile.tile_ic <= 0 || e.tile.oc_per_wave <= 0) return false;
+  shape.stages = ceil_div(e.C, e.tile.tile_ic);
+  shape.slots = ceil_div(e.K, kSlotPad) * kSlotPad;
+  Geom g;
+  return make_geom(&shape, e.N, e.H, e.W, e.stride, e.pad, e.tile, &g) == TETRIS_OK;
+}
+
+bool same_shape(const Tuned& e, int N, int H, int W, int C, int K, int ks, int stride, int pad) {
+  return e.N == N && e.H == H && e.W == W && e.C == C && e.K == K && e.ks == ks && e.stride == stride && e.pad == pad;
+}
 }  // namespace
 
+int load_tile_table(const char* path, int* rows_out) {
+  FILE* fp = std::fopen(path, "r");
+  if (!fp) return fail(TETRIS_EIO, "cannot open tile table %s", path);
+  std::vector<Tuned> rows;
+  char line[512];
+  while (std::fgets(line, sizeof line, fp)) {
+    Tuned e;
+    if (std::sscanf(line, " {%d, %d, %d, %d, %d, %d, %d, %d, {%d, %d, %d, %d, %d}}", &e.N, &e.H, &e.W, &e.C, &e.K, &e.ks,
+                    &e.stride, &e.pad, &e.tile.lanes_w, &e.tile.quads, &e.tile.oc_per_wave, &e.tile.waves,
+                    &e.tile.tile_ic) == 13)
+      rows.push_back(e);
+  }
+  std::fclose(fp);
+  std::lock_guard<std::mutex> lock(g_loaded_mu);
+  g_loaded.insert(g_loaded.begin(), rows.begin(), rows.end());
+  if (rows_out) *rows_out = (int)rows.size();
+  return TETRIS_OK;
+}
+
 int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t) {
+  {
+    std::lock_guard<std::mutex> lock(g_loaded_mu);
+    for (const Tuned& e : g_loaded)
+      if (same_shape(e, N, H, W, C, K, ks, stride, pad) && usable(e)) {
+        *t = e.tile;
+        return TETRIS_OK;
+      }
+  }
   for (const Tuned& e : kTuned)
-    if (e.N == N && e.H == H && e.W == W && e.C == C && e.K == K && e.ks == ks && e.stride == stride && e.pad == pad) {
-      // trust the table only as far as the kernel's own checks go
-      tetris_g950 shape;
-      shape.C = C; shape.K = K; shape.ks = ks; shape.tile_ic = e.tile.tile_ic; shape.g = e.tile.oc_per_wave;
-      shape.stages = ceil_div(C, e.tile.tile_ic);
-      shape.slots = ceil_div(K, kSlotPad) * kSlotPad;
-      Geom g;
-      if (make_geom(&shape, N, H, W, stride, pad, e.tile, &g) == TETRIS_OK) {
+    if (same_shape(e, N, H, W, C, K, ks, stride, pad)) {
+      if (usable(e)) {
         *t = e.tile;
         return TETRIS_OK;
       }

@@ -97,6 +97,7 @@ _lib.tetris_g950_destroy.argtypes = [C.c_void_p]
 _lib.tetris_g950_destroy.restype = None
 _lib.tetris_g950_host_arrays.argtypes = [C.c_void_p, C.POINTER(_G950Arrays)]
 _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
+_lib.tetris_tile_table_load.argtypes = [C.c_char_p, C.POINTER(C.c_int)]
 _lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(Tile),
                                           np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")]
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
@@ -262,6 +263,14 @@ def tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, strid
     _check(_lib.tetris_tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
                                    C.byref(t)))
     return t
+
+
+def tile_table_load(path):
+    """Makes tile_select answer from the rows of `path` (format of csrc/tuned_tiles.inc, written by tetris_amd.tune)
+    before the built-in table; -> number of rows read."""
+    n = C.c_int()
+    _check(_lib.tetris_tile_table_load(os.fsencode(path), C.byref(n)))
+    return int(n.value)
 
 
 def oc_order_balanced(filter, tile):
