@@ -150,8 +150,10 @@ int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int i
  * d_input is NCHW [batch][in_channel][img_h][img_w], d_output NCHW [batch][out_channel][oh][ow] with
  * oh = (img_h + 2*padding - kernel_size)/stride + 1 (the reference keeps NHWC on the device; its host
  * entry points below take and return NCHW, as here).  A layer with very few pixels per image is computed
- * by several workgroups per output tile: the launch then zero-fills d_output with a kernel of its own and the
- * workgroups add their partial sums with fp32 atomics, so the last bits can differ from run to run.
+ * by several workgroups per output tile: each writes partial sums to a scratch buffer owned by `p` (allocated or
+ * grown on the first such launch, freed with `p`) and a second kernel of the same launch adds them, in a fixed
+ * order, into d_output.  Launches of one pack that overlap in time on different streams share that scratch:
+ * give concurrent streams a pack each.
  * ---------------------------------------------------------------------------------------------- */
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
                            int stride, int padding, const tetris_tile* tile, void* stream);

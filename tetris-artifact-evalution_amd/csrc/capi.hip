@@ -78,7 +78,21 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
       if (p->plans.size() < 64) p->plans.push_back(plan);
     }
   }
-  return launch_conv(plan.geom, d_in, d_out, plan.entries, p->d_grp_off, p->d_oc_order, stream);
+  float* d_partial = nullptr;
+  if (plan.geom.csplit > 1) {
+    const Geom& g = plan.geom;
+    const size_t need = sizeof(float) * (size_t)g.csplit * g.N * g.K * g.OH * g.OW;
+    std::lock_guard<std::mutex> lock(p->mu);
+    if (p->partial_bytes < need) {
+      if (p->d_partial) TETRIS_HIP(hipFree(p->d_partial));  // waits for launches that still use it
+      p->d_partial = nullptr;
+      p->partial_bytes = 0;
+      TETRIS_HIP(hipMalloc(&p->d_partial, need));
+      p->partial_bytes = need;
+    }
+    d_partial = p->d_partial;
+  }
+  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, p->d_grp_off, p->d_oc_order, stream);
 }
 
 int time_launches(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,

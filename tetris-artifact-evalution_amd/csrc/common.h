@@ -41,6 +41,7 @@ constexpr int kMaxChunks16 = 6;
 //      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
 constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4 * quads
 constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
+constexpr int kMaxSplit = 8;      // most workgroups that may share an output tile (each reduces a slice of the stages)
 
 inline int out_extent(int in, int pad, int ks, int stride) { return (in + 2 * pad - ks) / stride + 1; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -91,8 +92,8 @@ struct Geom {
   int ver;             // 2: single LDS tile, register staging; 3: three LDS buffers, direct-to-LDS staging
   int cpp, nchunks, ni;
   int buf_bytes;       // size of one of the three LDS buffers: kBufBytes, or kHalfBufBytes (8 waves of <= 64 accumulators)
-  int csplit;          // workgroups that share an output tile, each reducing a slice of the stages and adding its
-                       // partial sums to the (pre-zeroed) output with atomics; 1 = plain stores
+  int csplit;          // workgroups that share an output tile, each reducing a slice of the stages into its own copy
+                       // of the output (a scratch buffer); reduce_kernel adds the copies.  1 = no split
   int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
@@ -141,6 +142,9 @@ struct tetris_g950 {
   // (LDS byte offset | accumulator index << 16 | 0xC << 28, value) pairs for one tile geometry, made on first use
   std::map<tetris::BoundKey, int2*> bound;
   std::vector<tetris::Plan> plans;  // few per pack; searched linearly, most recent first
+  // partial sums of layers whose channel reduction is split over workgroups: [csplit][N][K][OH][OW], grown on demand
+  float* d_partial = nullptr;
+  size_t partial_bytes = 0;
   std::mutex mu;
   // host mirrors, filled by tetris_g950_host_arrays
   std::vector<int32_t> h_grp_off, h_grp_nnz, h_position, h_oc_order;
@@ -180,9 +184,10 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
 int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_tile& t, int32_t* order);
 
 // spconv2d_kernel.hip
-// launches the conv (after a zero fill of the output when the geometry splits the channel reduction)
-int launch_conv(const Geom& g, const float* d_in, float* d_out, const int2* entries, const int32_t* grp_off,
-                const int32_t* oc_order, hipStream_t stream);
+// launches the conv; when the geometry splits the channel reduction (csplit > 1) the workgroups write their partial
+// sums to d_partial ([csplit] outputs) and a second kernel adds the slices, in order, into d_out
+int launch_conv(const Geom& g, const float* d_in, float* d_out, float* d_partial, const int2* entries,
+                const int32_t* grp_off, const int32_t* oc_order, hipStream_t stream);
 
 }  // namespace tetris
 

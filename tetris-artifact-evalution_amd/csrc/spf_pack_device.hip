@@ -246,6 +246,7 @@ void tetris_g950_destroy(tetris_g950* p) {
   (void)hipFree(p->d_position);
   (void)hipFree(p->d_values);
   (void)hipFree(p->d_oc_order);
+  (void)hipFree(p->d_partial);
   delete p;
 }
 

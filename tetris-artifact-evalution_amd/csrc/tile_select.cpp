@@ -143,7 +143,7 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     const long long room = 256ll * (g.ver == 3 && four ? 16 : 8);
     const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
     g.csplit = 1;
-    while (g.csplit < 8 && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
+    while (g.csplit < kMaxSplit && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
     if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32))
       return fail(TETRIS_EINVAL, "grid too large");
     g.m_kblocks = magic_reciprocal(g.kblocks);
