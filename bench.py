@@ -25,7 +25,7 @@ PEAK_FP32_TFLOPS = 157.3     # MI355X published vector/matrix fp32 peak
 
 # HBM bytes per launch of spconv2d_kernel (average over a step) from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
 # runs of this file, scaled by the same counters on a copy kernel of known size; see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.123e8}  # average per launch over the 16 layers
+MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.226e8}  # average per launch over the 16 layers
 
 
 def main():
