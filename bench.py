@@ -23,9 +23,10 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 PEAK_HBM_GBS = 8000.0        # MI355X published HBM3E bandwidth
 PEAK_FP32_TFLOPS = 157.3     # MI355X published vector/matrix fp32 peak
 
-# HBM bytes per launch of spconv2d_kernel (average over a step) from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`
-# runs of this file, scaled by the same counters on a copy kernel of known size; see profiles/.  None until measured.
-MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.226e8}  # average per launch over the 16 layers
+# HBM bytes per layer launch (spconv2d_kernel plus, for split layers, reduce_kernel; average over a step) from
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file, scaled by the same counters on a copy kernel of
+# known size; see profiles/.  None for workloads that were not measured.
+MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.451e8, "mobilenet/16": 4.113e7, "resnet50/16": 5.173e7}
 
 
 def main():
