@@ -46,8 +46,11 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
   const bool given = tile && tile->lanes_w > 0;
   Plan plan;
   bool found = false;
-  if (given) {
-    const int key[10] = {N, H, W, stride, pad, tile->lanes_w, tile->quads, tile->oc_per_wave, tile->waves, tile->tile_ic};
+  // a NULL tile is remembered under a key of zeros, so that the library's own choice is made once per shape
+  const tetris_tile none{};
+  const tetris_tile& kt = given ? *tile : none;
+  const int key[10] = {N, H, W, stride, pad, kt.lanes_w, kt.quads, kt.oc_per_wave, kt.waves, kt.tile_ic};
+  {
     std::lock_guard<std::mutex> lock(p->mu);
     for (size_t i = p->plans.size(); i-- > 0;)
       if (memcmp(p->plans[i].key, key, sizeof key) == 0) {
@@ -71,12 +74,9 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
     if (rc) return rc;
     rc = g950_bind(p, plan.geom, stream, &plan.entries);
     if (rc) return rc;
-    const int key[10] = {N, H, W, stride, pad, t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic};
     memcpy(plan.key, key, sizeof key);
-    if (given) {
-      std::lock_guard<std::mutex> lock(p->mu);
-      if (p->plans.size() < 64) p->plans.push_back(plan);
-    }
+    std::lock_guard<std::mutex> lock(p->mu);
+    if (p->plans.size() < 64) p->plans.push_back(plan);
   }
   float* d_partial = nullptr;
   if (plan.geom.csplit > 1) {
