@@ -111,7 +111,9 @@ typedef struct tetris_tile {
 } tetris_tile;
 
 /* Unmeasured selection: a built-in table of tiles measured on MI355X for the layer shapes of the benchmark
- * suites (csrc/tuned_tiles.inc, made by tetris_amd/tune.py), else the first choice of a cycle model. */
+ * suites (csrc/tuned_tiles.inc, made by tetris_amd/tune.py); for other shapes the tile of the most similar
+ * measured layer of the same kernel size and stride, refitted to the image width; else the first choice of a
+ * cycle model. */
 int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_channel, int kernel_size, int stride,
                        int padding, tetris_tile* out);
 

@@ -208,3 +208,18 @@ def test_tile_table_loaded_at_run_time_wins_over_the_built_in_one(tmp_path):
     with pytest.raises(T.TetrisError) as e:
         T.tile_table_load(str(tmp_path / "missing"))
     assert e.value.code == T.EIO
+
+
+def test_tile_select_borrows_from_the_nearest_measured_layer():
+    # a VGG19 layer shape at a batch size the table does not hold gets a measured neighbour's tile, not the cycle model's
+    t6 = T.tile_select(6, 56, 56, 256, 256, 3, 1, 1)
+    near = [T.tile_select(n, 56, 56, 256, 256, 3, 1, 1) for n in (4, 8)]
+    as_tuple = lambda t: (t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic)
+    assert as_tuple(t6) in [as_tuple(t) for t in near]
+    # the neighbour's lane count is refitted to the image width: a 52-wide layer is not given 14 lanes (two units per row)
+    t52 = T.tile_select(16, 52, 52, 256, 256, 3, 1, 1)
+    t50 = T.tile_select(16, 50, 50, 256, 256, 3, 1, 1)
+    assert -(-50 // (4 * t50.lanes_w)) == -(-52 // (4 * t52.lanes_w)) and 4 * t50.lanes_w - 50 < 4
+    # a kernel size no measured layer has falls through to the model and still gets a launchable tile
+    t5 = T.tile_select(2, 20, 20, 32, 32, 5, 1, 2)
+    assert t5.lanes_w >= 1 and t5.waves in (1, 2, 4, 8, 16)
