@@ -316,3 +316,12 @@ def test_tile_from_a_table_loaded_at_run_time(env, tmp_path):
     pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
     y = run_conv(T, torch, pk, x, K, ks, 1, 1, None)  # NULL tile: the library chooses, from the loaded row
     assert max_rel_err(y, O.host_conv2d(x, w, 1, 1, threads=4)) <= TOL
+
+
+def test_smoke_entry_point(env):
+    import importlib
+    import sys
+
+    from conftest import ROOT
+    sys.path.insert(0, ROOT)
+    importlib.import_module("__graft_entry__").smoke()
