@@ -325,3 +325,21 @@ def test_smoke_entry_point(env):
     from conftest import ROOT
     sys.path.insert(0, ROOT)
     importlib.import_module("__graft_entry__").smoke()
+
+
+def test_split_layers_are_bit_reproducible(env):
+    # A 14x14 layer whose channel reduction is split over workgroups: the partial sums are added in a fixed order,
+    # so two launches give the same bits, and a pack reused for a second shape regrows its scratch correctly.
+    T, torch, O = env
+    rng = np.random.default_rng(11)
+    C, K, ks = 512, 256, 1
+    w = sparse_filter(rng, K, C, ks, 0.85)
+    tile = T.tile_select(16, 14, 14, C, K, ks, 1, 0)  # one pack (tile) for all three launches
+    pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+    for N in (4, 16, 4):
+        x = relu_like(rng, (N, C, 14, 14))
+        a = run_conv(T, torch, pk, x, K, ks, 1, 0, tile)
+        b = run_conv(T, torch, pk, x, K, ks, 1, 0, tile)
+        assert a.tobytes() == b.tobytes()
+        assert max_rel_err(a, O.host_conv2d(x, w, 1, 0, threads=8)) <= TOL
+    pk.close()
