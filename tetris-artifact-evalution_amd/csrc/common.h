@@ -94,6 +94,10 @@ struct Geom {
   int buf_bytes;       // size of one of the three LDS buffers: kBufBytes, or kHalfBufBytes (8 waves of <= 64 accumulators)
   int csplit;          // workgroups that share an output tile, each reducing a slice of the stages into its own copy
                        // of the output (a scratch buffer); reduce_kernel adds the copies.  1 = no split
+  // A 1x1 convolution of stride s without padding only reads every s-th row and column: it is run as a stride-1
+  // layer on that sub-grid (H, W, stride above then describe the sub-grid) and the staging loads step through the
+  // real image: element (row, col) of the sub-grid lies at row*step*in_w + col*step of a plane of in_hw floats.
+  int step, in_w, in_hw;
   int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;

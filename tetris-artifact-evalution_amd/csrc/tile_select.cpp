@@ -73,6 +73,13 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   Geom g{};
   if (N <= 0 || H <= 0 || W <= 0 || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad conv shape N=%d H=%d W=%d stride=%d pad=%d", N, H, W, stride, pad);
+  g.step = 1; g.in_w = W; g.in_hw = H * W;
+  if (p->ks == 1 && stride > 1 && pad == 0) {  // only every stride-th row and column is read: stage just those
+    g.step = stride;
+    H = (H - 1) / stride + 1;
+    W = (W - 1) / stride + 1;
+    stride = 1;
+  }
   g.N = N; g.C = p->C; g.H = H; g.W = W; g.K = p->K; g.ks = p->ks; g.stride = stride; g.pad = pad;
   g.OH = out_extent(H, pad, p->ks, stride);
   g.OW = out_extent(W, pad, p->ks, stride);
@@ -118,7 +125,7 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   g.units = (int)units;
   g.ugroups = ceil_div(g.units, g.nq);
   // a workgroup addresses its images through one 2 GB buffer window
-  const long long img_bytes = 4ll * p->C * H * W;
+  const long long img_bytes = 4ll * p->C * g.in_hw;
   if (img_bytes * ((long long)g.nq * g.nb + 2) >= (1ll << 31))
     return fail(TETRIS_EINVAL, "images too large for the 2 GB input window of a workgroup");
   if ((long long)N * p->K * g.OH * g.OW >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
@@ -223,6 +230,11 @@ static int max_tile_ic(const Shape& s, int nq, int g, int waves, int stride, int
 int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad layer shape");
+  if (ks == 1 && stride > 1 && pad == 0) {  // run as a stride-1 layer on the sub-grid it reads (see make_geom)
+    H = (H - 1) / stride + 1;
+    W = (W - 1) / stride + 1;
+    stride = 1;
+  }
   const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
   if (OH <= 0 || OW <= 0) return fail(TETRIS_EINVAL, "empty output");
   // Score every candidate with a small time model calibrated on MI355X and keep the cheapest:
