@@ -192,4 +192,34 @@ inline bool TensorEqual(float* tensor_x, float* tensor_y, size_t len) {
   return true;
 }
 
+// Dense direct convolution on the host, for checking a result the way the reference's mains do when they are not
+// built for benchmarking (HostConv2d, Tetris/tensor_utils.cc:136-170; used at Tetris/spconv2d.cc:430-440): NCHW
+// input, OIHW filter, NCHW output, zero padding, every output summed over (ic, row, column) in that order.  It is a
+// checker: nothing in the library calls it.
+inline void HostConv2d(const float* input, const float* filter, float* output, int batch_size, int img_h, int img_w,
+                       int in_channel, int out_channel, int kernel_size, int stride, int padding) {
+  const int out_h = (img_h + 2 * padding - kernel_size) / stride + 1;
+  const int out_w = (img_w + 2 * padding - kernel_size) / stride + 1;
+  for (int n = 0; n < batch_size; ++n)
+    for (int k = 0; k < out_channel; ++k)
+      for (int oy = 0; oy < out_h; ++oy)
+        for (int ox = 0; ox < out_w; ++ox) {
+          float sum = 0.f;
+          for (int c = 0; c < in_channel; ++c) {
+            const float* plane = input + (static_cast<size_t>(n) * in_channel + c) * img_h * img_w;
+            const float* taps = filter + (static_cast<size_t>(k) * in_channel + c) * kernel_size * kernel_size;
+            for (int r = 0; r < kernel_size; ++r) {
+              const int iy = oy * stride - padding + r;
+              if (iy < 0 || iy >= img_h) continue;
+              for (int t = 0; t < kernel_size; ++t) {
+                const int ix = ox * stride - padding + t;
+                if (ix < 0 || ix >= img_w) continue;
+                sum += plane[iy * img_w + ix] * taps[r * kernel_size + t];
+              }
+            }
+          }
+          output[((static_cast<size_t>(n) * out_channel + k) * out_h + oy) * out_w + ox] = sum;
+        }
+}
+
 #endif  // TETRIS_SPCONV2D_HPP_

@@ -68,6 +68,19 @@ def test_cli_output_and_tensors(oracle, tmp_path, exe, shape):
 
 
 @pytest.mark.gpu
+def test_cli_check_option_prints_the_reference_verdict(tmp_path):
+    rng = np.random.default_rng(4)
+    w = sparse_filter(rng, 24, 16, 3, 0.8)
+    wf = str(tmp_path / "layer.txt")
+    write_weight_file(wf, w, 12, 12, 1, 1)
+    p = subprocess.run([os.path.join(BIN, "spconv2d_test"), wf, "2", "--check"], capture_output=True, text=True, timeout=120)
+    assert p.returncode == 0, p.stderr
+    lines = p.stdout.splitlines()
+    assert lines.index("HostConv2d begin") < lines.index("HostConv2d end") < lines.index("Sparse Pass.")
+    assert "Sparse Error." not in p.stdout
+
+
+@pytest.mark.gpu
 def test_cli_missing_file_behaves_like_the_reference():
     p = subprocess.run([os.path.join(BIN, "spconv2d_test"), "/nonexistent/layer", "1"], capture_output=True, text=True,
                        timeout=60)

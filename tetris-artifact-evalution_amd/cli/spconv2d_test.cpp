@@ -1,4 +1,4 @@
-// spconv2d_test <weight_file> [batch] [--seed S] [--dump FILE]      (built twice: spconv2d_test and, with
+// spconv2d_test <weight_file> [batch] [--seed S] [--dump FILE] [--check]      (built twice: spconv2d_test and, with
 // -DTETRIS_CLI_SPF, spf_test)
 //
 // Counterpart of the reference's per-layer binaries: main of Tetris/spconv2d.cc:369-450 (spconv2d_test.o,
@@ -12,7 +12,8 @@
 // seeded generator so that a run can be repeated, and --dump writes input and output tensors (raw
 // fp32: N*C*H*W inputs, then N*K*OH*OW outputs, both NCHW) for an external checker.  Like the
 // reference's shipped builds (BENCHMARK is defined in Tetris/tensor_utils.h:8) no CPU convolution is
-// run here.
+// run by default; --check does what the reference's other build does (Tetris/spconv2d.cc:430-440): a dense
+// convolution on the host, "HostConv2d begin" / "HostConv2d end", then "Sparse Pass." or "Sparse Error.".
 #include <hip/hip_runtime_api.h>
 
 #include <cassert>
@@ -62,6 +63,7 @@ int main(int argc, char* argv[]) {
   std::cout << "\n\n";
 
   std::string weight_file, dump;
+  bool check = false;
   int batch_size = 4;
   uint64_t seed = 1;
   int positional = 0;
@@ -70,6 +72,8 @@ int main(int argc, char* argv[]) {
       seed = std::strtoull(argv[++i], nullptr, 10);
     } else if (!std::strcmp(argv[i], "--dump") && i + 1 < argc) {
       dump = argv[++i];
+    } else if (!std::strcmp(argv[i], "--check")) {
+      check = true;
     } else if (positional == 0) {
       weight_file = argv[i];
       ++positional;
@@ -77,12 +81,12 @@ int main(int argc, char* argv[]) {
       batch_size = std::atoi(argv[i]);
       ++positional;
     } else {
-      std::fprintf(stderr, "usage: %s <weight_file> [batch] [--seed S] [--dump FILE]\n", argv[0]);
+      std::fprintf(stderr, "usage: %s <weight_file> [batch] [--seed S] [--dump FILE] [--check]\n", argv[0]);
       return 2;
     }
   }
   if (weight_file.empty() || batch_size <= 0) {
-    std::fprintf(stderr, "usage: %s <weight_file> [batch] [--seed S] [--dump FILE]\n", argv[0]);
+    std::fprintf(stderr, "usage: %s <weight_file> [batch] [--seed S] [--dump FILE] [--check]\n", argv[0]);
     return 2;
   }
 
@@ -122,6 +126,20 @@ int main(int argc, char* argv[]) {
                                     kernel_size, stride, padding, stream, layout, apply_reorder);
 #endif
   CLI_HIP(hipStreamDestroy(stream));
+
+  if (check) {  // what the reference's mains do when not built with -DBENCHMARK (Tetris/spconv2d.cc:430-440)
+    float* h_check = static_cast<float*>(std::malloc(n_out * sizeof(float)));
+    if (!h_check) {
+      std::fprintf(stderr, "out of host memory\n");
+      return 1;
+    }
+    std::cout << "HostConv2d begin\n";
+    HostConv2d(h_input, h_filter, h_check, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
+               padding);
+    std::cout << "HostConv2d end\n";
+    std::cout << (TensorEqual(h_sparse, h_check, n_out) ? "Sparse Pass.\n" : "Sparse Error.\n");
+    std::free(h_check);
+  }
 
   if (!dump.empty()) {
     FILE* fp = std::fopen(dump.c_str(), "wb");
