@@ -130,7 +130,8 @@ int tetris_tile_table_load(const char* path, int* rows_out);
  * (uses tile->oc_per_wave, waves and tile_ic).  Plays the part of SparseFilter::ReorderOutChannel
  * (Tetris/spconv2d_utils.h:275-420) for the HIP kernel: channels sorted by their non-zero count are dealt to the
  * workgroups' blocks of waves*oc_per_wave slots in serpentine order, then inside a block each goes to the wave
- * where it adds least to the sum over input-channel stages of the busiest wave's entries.  On pruned networks,
+ * where it adds least to the sum over input-channel stages of the busiest SIMD's entries (waves w, w+4, ... share
+ * a SIMD), then of the busiest wave's.  On pruned networks,
  * whose channels differ widely in density, the busiest wave of a stage holds 1.2-1.5x the mean in file order.
  * `order_out` receives a permutation of 0..out_channel-1.  Pure host code. */
 int tetris_oc_order_balanced(const float* h_filter_oihw, int in_channel, int out_channel, int kernel_size,
