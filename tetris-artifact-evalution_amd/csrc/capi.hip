@@ -342,7 +342,8 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
       it = packs.emplace(key, p).first;
     }
     float ms = 0;
-    rc = time_launches(it->second, d_in, d_out, N, H, W, stride, pad, &t, stream, 1, 3, &ms);
+    // the first candidate also warms the clocks up: a GPU that idled runs its first launches several per cent slow
+    rc = time_launches(it->second, d_in, d_out, N, H, W, stride, pad, &t, stream, timed.empty() ? 8 : 1, 3, &ms);
     if (rc == TETRIS_EINVAL) continue;  // the model ranks shapes make_geom may still refuse
     if (rc) return done(rc);
     timed.emplace_back(ms, t);
