@@ -343,3 +343,49 @@ def test_split_layers_are_bit_reproducible(env):
         assert a.tobytes() == b.tobytes()
         assert max_rel_err(a, O.host_conv2d(x, w, 1, 0, threads=8)) <= TOL
     pk.close()
+
+
+def test_launches_can_be_captured_in_a_hip_graph(env):
+    # After one eager launch per shape (which makes the launch plan and, for a split layer, its scratch buffer) a
+    # launch is nothing but kernel launches on the caller's stream, so a chain of layers can be captured once and
+    # replayed.  Checked on three layers, one of them split over workgroups, over several replays with new inputs.
+    T, torch, O = env
+    rng = np.random.default_rng(21)
+    N = 4
+    specs = [(16, 28, 32, 3, 1, 1), (32, 28, 512, 1, 2, 0), (512, 14, 64, 1, 1, 0)]  # C, H, K, ks, stride, pad
+    ws, packs, tiles, bufs = [], [], [], []
+    x0 = torch.zeros((N, 16, 28, 28), device="cuda")
+    cur = x0
+    for C, H, K, ks, stride, pad in specs:
+        w = sparse_filter(rng, K, C, ks, 0.8)
+        tile = T.tile_select(N, H, H, C, K, ks, stride, pad)
+        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+        oh = T.out_extent(H, pad, ks, stride)
+        y = torch.empty((N, K, oh, oh), device="cuda")
+        ws.append(w); packs.append(pk); tiles.append(tile); bufs.append((cur, y, H, stride, pad))
+        cur = y
+
+    def run(stream):
+        for pk, tile, (xin, y, H, stride, pad) in zip(packs, tiles, bufs):
+            pk.launch(xin.data_ptr(), y.data_ptr(), N, H, H, stride, pad, tile, stream=stream)
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        run(side.cuda_stream)  # eager warm-up: plans, scratch
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(side.cuda_stream)
+    for rep in range(3):
+        x = relu_like(rng, (N, 16, 28, 28))
+        x0.copy_(torch.from_numpy(x))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ref = x
+        for w, (C, H, K, ks, stride, pad) in zip(ws, specs):
+            ref = O.host_conv2d(ref, w, stride, pad, threads=8)
+        got = bufs[-1][1].cpu().numpy()
+        assert max_rel_err(got, ref) <= 3 * TOL, rep  # three chained layers: errors of the first two feed the third
+    for pk in packs:
+        pk.close()
