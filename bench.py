@@ -213,6 +213,15 @@ def main():
                "kind": "port", "sample": "first %d of %d %s layers at batch %d (one pass), packed-format decode conv of the "
                "oracle (restates HostReorderSpconv2d, spconv2d_utils.h:457-493), OpenMP over (n, oc), %.1f s wall" % (
                    used, len(sample_layers), args.suite, N, t_cpu)}
+        # the dense CPU convolution of the same path (restates HostConv2d, tensor_utils.cc:136-170), OpenMP over (n, oc)
+        L = W.single_layer()[0]
+        w1, x4 = W.make_weights(L), W.make_activations(L, 4)
+        t0 = time.perf_counter()
+        O.host_conv2d(x4, w1, L.stride, L.pad, threads=threads)
+        dt = time.perf_counter() - t0
+        cpu["dense_host_conv2d"] = {"value": round(W.work(L, 4)["flops_dense"] / dt / 1e9, 2), "unit": "GFLOP/s",
+                                    "cores": threads, "kind": "port",
+                                    "sample": "single 64->128 56x56 3x3 layer, batch 4, %.2f s" % dt}
         if O.ref_available():
             L = W.single_layer()[0]
             w, x1 = W.make_weights(L), W.make_activations(L, 1)
