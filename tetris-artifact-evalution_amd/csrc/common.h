@@ -98,7 +98,7 @@ struct Geom {
   // layer on that sub-grid (H, W, stride above then describe the sub-grid) and the staging loads step through the
   // real image: element (row, col) of the sub-grid lies at row*step*in_w + col*step of a plane of in_hw floats.
   int step, in_w, in_hw;
-  int stagers;         // waves 0 .. stagers-1 fill LDS (all of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
+  int stagers;         // waves 0 .. stagers-1 fill LDS (4 or 8 of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan

@@ -159,10 +159,12 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   if (g.ver == 3) {
     g.cpp = ceil_div(g.plane, 64);
     g.nchunks = g.nq * g.nb * g.cpp;
-    // a 16-wave workgroup leaves the staging to its four oldest waves when they can hold the plan
+    // a workgroup of 8 or 16 waves leaves the staging to its four oldest waves when they can hold the plan (the
+    // hardware serves the oldest wave of a SIMD first: they finish their walk early and would idle at the barrier)
     g.stagers = t.waves;
     const int max_chunks = (t.waves == 16 || g.buf_bytes == kHalfBufBytes) ? kMaxChunks16 : kMaxChunks;
     if (t.waves == 16) g.stagers = g.nchunks <= 4 * max_chunks ? 4 : g.nchunks <= 8 * max_chunks ? 8 : 16;
+    if (t.waves == 8 && g.nchunks <= 4 * max_chunks) g.stagers = 4;
     g.ni = ceil_div(g.nchunks, g.stagers);
     if (64ll * (g.cpp + 1) * g.pitch >= (1ll << 32))
       return fail(TETRIS_EINVAL, "too many pixel units for the kernel's index arithmetic");
