@@ -290,7 +290,10 @@ def main():
         "ms_per_step_device": round(ms_per_step_dev, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s-shaped sparse conv stack, %d layers, batch %d, fp32 NCHW, seeded unstructured masks"
-                   % (args.suite, len(layers), N), "suite": args.suite, "batch": N, "layers": len(layers)},
+                   % (args.suite, len(layers), N), "suite": args.suite, "batch": N, "layers": len(layers),
+                   "base_seed": W.BASE_SEED,
+                   "tensor_seed": "base_seed ^ crc32('<suite>/<layer index>/<w|x>'), splitmix64 streams "
+                                  "(tetris_amd/workloads.py)"},
         "sparse_gflops": round(fl_sparse / (ms_per_step * 1e-3) / 1e9, 1),
         "sum_layer_us": round(t_layers * 1e6, 1) if table else None,
         "pack_ms_total": round(t_pack * 1e3, 2),
