@@ -232,7 +232,21 @@ def main():
                                            "unit": "GFLOP/s", "cores": 1, "kind": "reference",
                                            "sample": "single 64->128 56x56 3x3 layer, batch 1, %.2f s" % dt}
 
-    context = None
+    # what this box's HBM delivers to a plain copy (256 MiB read + 256 MiB written per pass), next to the nominal peak
+    n_copy = 64 << 20
+    src = torch.ones(n_copy, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    c0.record()
+    for _ in range(10):
+        dst.copy_(src)
+    c1.record()
+    torch.cuda.synchronize()
+    context = {"measured_copy_gbs": round(10 * 2 * 4 * n_copy / (c0.elapsed_time(c1) * 1e-3) / 1e9, 1),
+               "copy_note": "torch copy of 256 MiB, read + write bytes over device time; nominal HBM peak 8000 GB/s"}
+    del src, dst
     if args.dense_baseline:
         import torch.nn.functional as F
         ws = [torch.from_numpy(W.make_weights(L)).to(dev) for L in layers]
@@ -251,14 +265,13 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         dense_ms = e0.elapsed_time(e1) / args.steps
-        context = {"vendor_dense_fp32_ms_per_step": round(dense_ms, 4),
+        context.update({"vendor_dense_fp32_ms_per_step": round(dense_ms, 4),
                    "vendor_dense_fp32_gflops": round(fl_dense / (dense_ms * 1e-3) / 1e9, 1),
                    "speedup_over_vendor_dense": round(dense_ms / ms_per_step, 3),
-                   "note": "torch.nn.functional.conv2d (MIOpen) on the same tensors, weights dense with the zeros in"}
+                   "note": "torch.nn.functional.conv2d (MIOpen) on the same tensors, weights dense with the zeros in"})
 
     if args.csr_baseline:
         import torch.nn.functional as F
-        context = context or {}
         try:
             csr = [torch.from_numpy(W.make_weights(L).reshape(L.K, -1)).to(dev).to_sparse_csr() for L in layers]
 
