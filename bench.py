@@ -232,21 +232,13 @@ def main():
                                            "unit": "GFLOP/s", "cores": 1, "kind": "reference",
                                            "sample": "single 64->128 56x56 3x3 layer, batch 1, %.2f s" % dt}
 
-    # what this box's HBM delivers to a plain copy (256 MiB read + 256 MiB written per pass), next to the nominal peak
-    n_copy = 64 << 20
-    src = torch.ones(n_copy, dtype=torch.float32, device=dev)
-    dst = torch.empty_like(src)
-    for _ in range(3):
-        dst.copy_(src)
-    c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    c0.record()
-    for _ in range(10):
-        dst.copy_(src)
-    c1.record()
-    torch.cuda.synchronize()
-    context = {"measured_copy_gbs": round(10 * 2 * 4 * n_copy / (c0.elapsed_time(c1) * 1e-3) / 1e9, 1),
-               "copy_note": "torch copy of 256 MiB, read + write bytes over device time; nominal HBM peak 8000 GB/s"}
-    del src, dst
+    # what this box delivers to a plain copy and to a loop of independent FMAs, next to the nominal peaks
+    copy_gbs, fma_tflops = T.measure_peaks()
+    context = {"measured_copy_gbs": round(copy_gbs, 1), "measured_fma_tflops": round(fma_tflops, 2),
+               "peaks_note": "tetris_measure_peaks: device copy of 256 MiB (read + write bytes) and sixteen independent "
+                             "non-packed fp32 FMA chains per lane; nominal peaks 8000 GB/s and 157.3 TFLOP/s (packed)",
+               "roofline_frac_of_measured": round((fl_sparse / t_step / 1e12) / fma_tflops, 4) if t_fp32 >= t_hbm
+               else round((bytes_alg / t_step / 1e9) / copy_gbs, 4)}
     if args.dense_baseline:
         import torch.nn.functional as F
         ws = [torch.from_numpy(W.make_weights(L)).to(dev) for L in layers]

@@ -126,6 +126,13 @@ int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_
  * Process-wide; may be called several times (later files win). */
 int tetris_tile_table_load(const char* path, int* rows_out);
 
+/* What this GPU delivers to a plain device copy (GB/s, read + write bytes of a 256 MiB buffer) and to a loop of
+ * independent fp32 FMAs (TFLOP/s, non-packed), for reading roofline fractions against measured ceilings as well
+ * as nominal ones.  No reference counterpart (the reference prints milliseconds and "T" per layer only,
+ * Tetris/spconv2d.cc:357-358).  Allocates 512 MiB for its duration; synchronises `stream`.  Either output may
+ * be NULL. */
+int tetris_measure_peaks(void* stream, float* copy_gbs_out, float* fma_tflops_out);
+
 /* Output-channel order for tetris_g950_create that evens out the work of the waves of a workgroup of `tile`
  * (uses tile->oc_per_wave, waves and tile_ic).  Plays the part of SparseFilter::ReorderOutChannel
  * (Tetris/spconv2d_utils.h:275-420) for the HIP kernel: channels sorted by their non-zero count are dealt to the

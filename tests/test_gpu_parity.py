@@ -389,3 +389,10 @@ def test_launches_can_be_captured_in_a_hip_graph(env):
         assert max_rel_err(got, ref) <= 3 * TOL, rep  # three chained layers: errors of the first two feed the third
     for pk in packs:
         pk.close()
+
+
+def test_measured_ceilings_are_plausible(env):
+    T, torch, O = env
+    copy_gbs, fma_tflops = T.measure_peaks()
+    assert 2000 < copy_gbs < 8000   # nominal HBM peak 8000 GB/s
+    assert 40 < fma_tflops < 157.3  # nominal 157.3 TFLOP/s needs packed fp32; non-packed code can reach half of it

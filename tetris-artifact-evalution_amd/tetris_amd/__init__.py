@@ -98,6 +98,7 @@ _lib.tetris_g950_destroy.restype = None
 _lib.tetris_g950_host_arrays.argtypes = [C.c_void_p, C.POINTER(_G950Arrays)]
 _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
 _lib.tetris_tile_table_load.argtypes = [C.c_char_p, C.POINTER(C.c_int)]
+_lib.tetris_measure_peaks.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
 _lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(Tile),
                                           np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")]
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
@@ -271,6 +272,13 @@ def tile_table_load(path):
     n = C.c_int()
     _check(_lib.tetris_tile_table_load(os.fsencode(path), C.byref(n)))
     return int(n.value)
+
+
+def measure_peaks(stream=0):
+    """-> (device copy GB/s, non-packed fp32 FMA TFLOP/s) measured on this GPU (tetris_measure_peaks)."""
+    c, f = C.c_float(), C.c_float()
+    _check(_lib.tetris_measure_peaks(C.c_void_p(stream), C.byref(c), C.byref(f)))
+    return float(c.value), float(f.value)
 
 
 def oc_order_balanced(filter, tile):
