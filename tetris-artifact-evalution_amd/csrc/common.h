@@ -98,11 +98,18 @@ struct Geom {
   // layer on that sub-grid (H, W, stride above then describe the sub-grid) and the staging loads step through the
   // real image: element (row, col) of the sub-grid lies at row*step*in_w + col*step of a plane of in_hw floats.
   int step, in_w, in_hw;
+  // Images side by side: a tile whose lanes span the image width twice or four times over (2*lw >= OW, lw >= OW)
+  // gives quads j = 0..3 of a lane to `fold` = 2 or 4 different images instead of to four column groups of one:
+  // quad j belongs to image j >> jsh of the unit and to column group j & ((1 << jsh) - 1).  fold = 1, jsh = 2 otherwise.
+  int fold, jsh;
   int stagers;         // waves 0 .. stagers-1 fill LDS (4 or 8 of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan
 };
+
+// how many images a tile of `lw` lanes per row places side by side on an output OW pixels wide
+inline int fold_of(int lw, int OW) { return lw >= OW ? 4 : 2 * lw >= OW ? 2 : 1; }
 
 // Byte offset that the packed entry (ic_local, r, s) adds to a lane's LDS base address.
 inline int lds_entry_offset(int plane, int pitch, int par, int stride, int ic_local, int r, int s) {

@@ -102,7 +102,9 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   if (g.g * 4 * g.nq > acc_regs)
     return fail(TETRIS_EINVAL, "oc_per_wave * 4 * quads = %d exceeds the %d accumulators of a wave", g.g * 4 * g.nq,
                 acc_regs);
-  const Shape s = unit_shape(t.lanes_w, g.OH, N, p->ks, stride);
+  g.fold = fold_of(t.lanes_w, g.OW);
+  g.jsh = g.fold == 4 ? 0 : g.fold == 2 ? 1 : 2;
+  const Shape s = unit_shape(t.lanes_w, g.OH, ceil_div(N, g.fold), p->ks, stride);
   g.lw = s.lw; g.lr = s.lr; g.lh = s.lh; g.thi = s.thi; g.nb = s.nb; g.ng = s.ng; g.par = s.par; g.ih = s.ih;
   g.ver = t.waves >= 8 ? 3 : 2;
   // 8 waves that need at most 64 accumulators each leave room for a second workgroup on the CU
@@ -114,9 +116,9 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   if (4ll * g.nb * g.img_stride > g.region)
     return fail(TETRIS_EINVAL, "a pixel unit needs %lld bytes of LDS for %d staged channels (region is %d): lower tile_ic "
                 "or quads", 4ll * g.nb * g.img_stride, g.tile_ic, g.region);
-  g.units_w = ceil_div(g.OW, 4 * g.lw);
+  g.units_w = ceil_div(g.OW, (4 / g.fold) * g.lw);
   g.units_h = ceil_div(g.OH, g.thi);
-  g.units_n = ceil_div(N, g.nb);
+  g.units_n = ceil_div(N, g.nb * g.fold);
   const long long units = (long long)g.units_w * g.units_h * g.units_n;
   g.kb = t.waves * g.g;
   g.kblocks = ceil_div(p->K, g.kb);
@@ -126,11 +128,11 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   g.ugroups = ceil_div(g.units, g.nq);
   // a workgroup addresses its images through one 2 GB buffer window
   const long long img_bytes = 4ll * p->C * g.in_hw;
-  if (img_bytes * ((long long)g.nq * g.nb + 2) >= (1ll << 31))
+  if (img_bytes * ((long long)g.nq * g.nb * g.fold + 2) >= (1ll << 31))
     return fail(TETRIS_EINVAL, "images too large for the 2 GB input window of a workgroup");
   if ((long long)N * p->K * g.OH * g.OW >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
   // ... and writes its outputs through one as well
-  if (4ll * p->K * g.OH * g.OW * ((long long)g.nq * g.nb + 2) >= (1ll << 31))
+  if (4ll * p->K * g.OH * g.OW * ((long long)g.nq * g.nb * g.fold + 2) >= (1ll << 31))
     return fail(TETRIS_EINVAL, "images too large for the 2 GB output window of a workgroup");
   // staging plan
   g.slots_per_unit = g.nb * g.ih * stride * g.ng;
@@ -249,10 +251,14 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
   const double density = 0.15;  // the mask is not known here; typical of the pruned layers this runs
   std::vector<std::pair<double, tetris_tile>> scored;
   for (int lw = 1; lw <= 62; ++lw) {
-    if (4 * (lw - 1) >= OW && lw > 1) break;  // wider than the image
+    if (lw > OW && lw > 1) break;  // wider than four images side by side could use
     if (4 * lw < (OW >= 28 ? 28 : (OW + 1) / 2)) continue;  // narrow tiles stage their halo'd rows poorly (measured)
-    const Shape s = unit_shape(lw, OH, N, ks, stride);
-    const long long units = (long long)ceil_div(OW, 4 * lw) * ceil_div(OH, s.thi) * ceil_div(N, s.nb);
+    const int fold = fold_of(lw, OW);
+    // wider than the image only to place 2 or 4 images side by side, and then only as wide as that needs
+    if (4 * (lw - 1) >= OW && lw > 1 && (fold == 1 || N < fold || (fold == 2 && 2 * (lw - 1) >= OW) || (fold == 4 && lw - 1 >= OW)))
+      continue;
+    const Shape s = unit_shape(lw, OH, ceil_div(N, fold), ks, stride);
+    const long long units = (long long)ceil_div(OW, (4 / fold) * lw) * ceil_div(OH, s.thi) * ceil_div(N, s.nb * fold);
     for (const auto& qg : kQuadG) {
       const int nq = qg[0], g = qg[1];
       for (int waves : kWaves) {
@@ -379,8 +385,10 @@ int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, 
     for (size_t i = 0; i < near.size() && i < 6 && near[i].first < 6.0; ++i) {
       Tuned cand = *near[i].second;
       // same number of units across the image as in the neighbour, at this image's width
-      const int units_w = ceil_div(out_extent(cand.W, cand.pad, cand.ks, cand.stride), 4 * cand.tile.lanes_w);
-      cand.tile.lanes_w = ceil_div(OW, 4 * units_w);
+      const int eow = out_extent(cand.W, cand.pad, cand.ks, cand.stride);
+      const int per_image = 4 / fold_of(cand.tile.lanes_w, eow);  // column groups of a lane that belong to one image
+      const int units_w = ceil_div(eow, per_image * cand.tile.lanes_w);
+      cand.tile.lanes_w = ceil_div(OW, per_image * units_w);
       cand.N = N; cand.H = H; cand.W = W; cand.C = C; cand.K = K; cand.pad = pad;
       cand.tile.tile_ic = std::min(cand.tile.tile_ic, C);
       if (usable(cand)) {
