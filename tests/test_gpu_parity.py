@@ -396,3 +396,29 @@ def test_measured_ceilings_are_plausible(env):
     copy_gbs, fma_tflops = T.measure_peaks()
     assert 2000 < copy_gbs < 8000   # nominal HBM peak 8000 GB/s
     assert 40 < fma_tflops < 157.3  # nominal 157.3 TFLOP/s needs packed fp32; non-packed code can reach half of it
+
+
+@pytest.mark.parametrize("case", [
+    # N, C, H, W, K, ks, stride, pad, (lanes_w, quads, oc_per_wave, waves, tile_ic)
+    (5, 24, 14, 14, 40, 3, 1, 1, (7, 1, 8, 4, 8)),     # two images side by side, odd batch: the last pair is half empty
+    (5, 24, 14, 14, 40, 3, 1, 1, (14, 2, 8, 16, 8)),   # four side by side, 16 waves
+    (3, 16, 28, 28, 32, 3, 1, 1, (14, 2, 8, 8, 8)),    # the 28x28 case of the VGG19 stack
+    (6, 32, 13, 13, 64, 3, 2, 1, (7, 1, 4, 4, 4)),     # stride 2: parity planes, four side by side (OW = 7)
+    (7, 40, 7, 7, 72, 1, 1, 0, (7, 1, 8, 4, 16)),      # 7x7, 1x1: four side by side, rows of several images folded too
+    (4, 8, 10, 6, 16, 5, 1, 2, (3, 1, 4, 2, 4)),       # 5x5 kernel: a two-column halo at every seam
+])
+def test_images_side_by_side(env, case):
+    # Tiles at least twice as wide as the output give the quads of a lane to different images; the seams between the
+    # images must behave like image borders (zero padding), which a kernel wider than one column probes.
+    T, torch, O = env
+    N, C, H, W, K, ks, stride, pad, tile = case
+    tile = T.Tile(*tile)
+    ow = T.out_extent(W, pad, ks, stride)
+    assert 2 * tile.lanes_w >= ow  # the tile folds
+    rng = np.random.default_rng(N * 100 + W)
+    w = sparse_filter(rng, K, C, ks, 0.6)
+    x = relu_like(rng, (N, C, H, W)) + 0.25  # no zeros near the borders: a wrong seam would show
+    pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+    y = run_conv(T, torch, pk, x.astype(np.float32), K, ks, stride, pad, tile)
+    assert max_rel_err(y, O.host_conv2d(x.astype(np.float32), w, stride, pad, threads=4)) <= TOL
+    pk.close()
