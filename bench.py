@@ -26,7 +26,7 @@ PEAK_FP32_TFLOPS = 157.3     # MI355X published vector/matrix fp32 peak
 # HBM bytes per layer launch (spconv2d_kernel plus, for split layers, reduce_kernel; average over a step) from
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file, scaled by the same counters on a copy kernel of
 # known size; see profiles/.  None for workloads that were not measured.
-MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.456e8, "mobilenet/16": 4.114e7, "resnet50/16": 4.855e7}
+MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.478e8, "mobilenet/16": 4.016e7, "resnet50/16": 5.056e7}
 
 
 def main():
