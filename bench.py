@@ -32,8 +32,8 @@ MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.478e8, "mobilenet/16": 4.016e7, "resnet5
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--suite", default="vgg19")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--masks", metavar="NPZ", help="run the layers of a pruned network instead of --suite: a mask file "
