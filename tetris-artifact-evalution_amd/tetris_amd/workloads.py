@@ -24,13 +24,16 @@ _M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
 BASE_SEED = 0x7E7A15
 
 
-def _splitmix64(seed, n):
-    """n outputs of splitmix64 started at `seed` (vectorised: output i hashes seed + (i+1)*gamma)."""
+def _splitmix64(seed, n, start=0):
+    """Outputs start .. start+n-1 of splitmix64 started at `seed` (vectorised: output i hashes seed + (i+1)*gamma)."""
     with np.errstate(over="ignore"):
-        z = np.uint64(seed) + (np.arange(1, n + 1, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
-        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
-        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
-        return z ^ (z >> np.uint64(31))
+        z = np.uint64(seed) + (np.arange(start + 1, start + n + 1, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
+        z ^= z >> np.uint64(30)
+        z *= np.uint64(0xBF58476D1CE4E5B9)
+        z ^= z >> np.uint64(27)
+        z *= np.uint64(0x94D049BB133111EB)
+        z ^= z >> np.uint64(31)
+        return z
 
 
 def tensor_seed(suite, index, kind, base_seed=BASE_SEED):
@@ -59,9 +62,14 @@ def make_weights(layer, base_seed=BASE_SEED):
 def make_activations(layer, batch, base_seed=BASE_SEED):
     n = batch * layer.C * layer.H * layer.W
     seed = tensor_seed(layer.suite, layer.index, "x", base_seed)
-    bits = _splitmix64(seed, n)
-    x = ((bits >> np.uint64(40)).astype(np.float32) * np.float32(1.0 / (1 << 24)))
-    x[(bits & np.uint64(1)) == 0] = 0.0
+    x = np.empty(n, np.float32)
+    chunk = 1 << 18  # cache-sized pieces: the same values several times faster than one pass over the whole tensor
+    for lo in range(0, n, chunk):
+        bits = _splitmix64(seed, min(chunk, n - lo), lo)
+        v = (bits >> np.uint64(40)).astype(np.float32)
+        v *= np.float32(1.0 / (1 << 24))
+        v[(bits & np.uint64(1)) == 0] = 0.0
+        x[lo:lo + len(v)] = v
     return x.reshape(batch, layer.C, layer.H, layer.W)
 
 
