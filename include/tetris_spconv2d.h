@@ -161,13 +161,23 @@ int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int i
  * d_input is NCHW [batch][in_channel][img_h][img_w], d_output NCHW [batch][out_channel][oh][ow] with
  * oh = (img_h + 2*padding - kernel_size)/stride + 1 (the reference keeps NHWC on the device; its host
  * entry points below take and return NCHW, as here).  A layer with very few pixels per image is computed
- * by several workgroups per output tile: each writes partial sums to a scratch buffer owned by `p` (allocated or
- * grown on the first such launch, freed with `p`) and a second kernel of the same launch adds them, in a fixed
- * order, into d_output.  Launches of one pack that overlap in time on different streams share that scratch:
- * give concurrent streams a pack each.
+ * by several workgroups per output tile: each writes partial sums to a scratch buffer owned by `p` and a second
+ * kernel of the same launch adds them, in a fixed order, into d_output.  `p` keeps one such buffer per stream it is
+ * launched on (made by tetris_g950_prepare or by the first such launch on that stream, freed with `p`), so launches
+ * of one pack on different streams do not disturb each other; two launches on ONE stream are ordered by the stream.
+ * The first launch of an (input shape, tile) pair also makes its launch plan (a device allocation and a small
+ * kernel); it is refused with TETRIS_EINVAL while `stream` is being captured -- call tetris_g950_prepare before.
  * ---------------------------------------------------------------------------------------------- */
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
                            int stride, int padding, const tetris_tile* tile, void* stream);
+
+/* Makes everything tetris_spconv2d_launch would otherwise make on its first call for (input shape, tile) on
+ * `stream`: the launch plan, the entries bound to the tile geometry and, for a split layer, the partial-sum buffer of
+ * that stream.  After it returns, launches with the same arguments allocate nothing and can be captured into a HIP
+ * graph.  Counterpart of the reference doing all its allocation in the SparseFilter constructor
+ * (Tetris/spconv2d_utils.h:248-264) before the launcher runs. */
+int tetris_g950_prepare(tetris_g950* p, int batch, int img_h, int img_w, int stride, int padding,
+                        const tetris_tile* tile, void* stream);
 
 /* Same call shape as the reference launcher: the raw device arrays of a live tetris_spf (looked up by
  * `d_values`).  tile_h/tile_w are accepted for source compatibility and ignored. */

@@ -391,6 +391,38 @@ def test_launches_can_be_captured_in_a_hip_graph(env):
         pk.close()
 
 
+def test_prepare_then_capture_without_an_eager_launch(env):
+    # tetris_g950_prepare makes the plan and a split layer's scratch, so the very first launch can be a captured one;
+    # an unprepared launch under capture is refused instead of allocating (which would break the capture).
+    T, torch, O = env
+    rng = np.random.default_rng(22)
+    N, C, H, K = 4, 512, 14, 64
+    w = sparse_filter(rng, K, C, 1, 0.8)
+    tile = T.Tile(14, 1, 8, 4, 32)  # split over workgroups on this shape
+    pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+    other = T.G950Filter.for_tile(w, tile)
+    x = torch.zeros((N, C, H, H), device="cuda")
+    y = torch.empty((N, K, H, H), device="cuda")
+    side = torch.cuda.Stream()
+    pk.prepare(N, H, H, 1, 0, tile, stream=side.cuda_stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        pk.launch(x.data_ptr(), y.data_ptr(), N, H, H, 1, 0, tile, stream=side.cuda_stream)
+        with pytest.raises(T.TetrisError) as e:
+            other.launch(x.data_ptr(), y.data_ptr(), N, H, H, 1, 0, tile, stream=side.cuda_stream)
+        assert e.value.code == T.EINVAL and "prepare" in str(e.value)
+    for rep in range(3):
+        xn = relu_like(rng, (N, C, H, H))
+        x.copy_(torch.from_numpy(xn))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert max_rel_err(y.cpu().numpy(), O.host_conv2d(xn, w, 1, 0, threads=8)) <= TOL, rep
+    pk.close()
+    other.close()
+
+
 def test_measured_ceilings_are_plausible(env):
     T, torch, O = env
     copy_gbs, fma_tflops = T.measure_peaks()

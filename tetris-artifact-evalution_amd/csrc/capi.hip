@@ -40,12 +40,11 @@ int upload(const std::vector<T>& v, T** d) {
   return TETRIS_OK;
 }
 
-int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
-               const tetris_tile* tile, hipStream_t stream) {
-  if (!p || !d_in || !d_out) return fail(TETRIS_EINVAL, "null argument");
+// The launch plan of (input shape, tile) for pack `p`: looked up, or -- when `create` allows it -- made (geometry,
+// bound entries: one device allocation and one small kernel on `stream`) and remembered.
+int find_plan(tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile* tile, hipStream_t stream,
+              bool create, Plan* out) {
   const bool given = tile && tile->lanes_w > 0;
-  Plan plan;
-  bool found = false;
   // a NULL tile is remembered under a key of zeros, so that the library's own choice is made once per shape
   const tetris_tile none{};
   const tetris_tile& kt = given ? *tile : none;
@@ -54,43 +53,77 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
     std::lock_guard<std::mutex> lock(p->mu);
     for (size_t i = p->plans.size(); i-- > 0;)
       if (memcmp(p->plans[i].key, key, sizeof key) == 0) {
-        plan = p->plans[i];
-        found = true;
-        break;
+        *out = p->plans[i];
+        return TETRIS_OK;
       }
   }
-  if (!found) {
-    tetris_tile t{};
-    if (given) {
-      t = *tile;
-    } else {
-      int rc = choose_tile(N, H, W, p->C, p->K, p->ks, stride, pad, &t);
-      if (rc) return rc;
-    }
-    if (t.tile_ic != p->tile_ic || t.oc_per_wave != p->g)
-      return fail(TETRIS_EINVAL, "tile (tile_ic=%d, oc_per_wave=%d) does not match the pack (tile_ic=%d, oc_per_wave=%d)",
-                  t.tile_ic, t.oc_per_wave, p->tile_ic, p->g);
-    int rc = make_geom(p, N, H, W, stride, pad, t, &plan.geom);
+  if (!create)
+    return fail(TETRIS_ENOTFOUND, "no launch plan for N=%d H=%d W=%d stride=%d pad=%d with this tile: call "
+                "tetris_g950_prepare first", N, H, W, stride, pad);
+  tetris_tile t{};
+  if (given) {
+    t = *tile;
+  } else {
+    int rc = choose_tile(N, H, W, p->C, p->K, p->ks, stride, pad, &t);
     if (rc) return rc;
-    rc = g950_bind(p, plan.geom, stream, &plan.entries);
-    if (rc) return rc;
-    memcpy(plan.key, key, sizeof key);
-    std::lock_guard<std::mutex> lock(p->mu);
-    if (p->plans.size() < 64) p->plans.push_back(plan);
   }
+  if (t.tile_ic != p->tile_ic || t.oc_per_wave != p->g)
+    return fail(TETRIS_EINVAL, "tile (tile_ic=%d, oc_per_wave=%d) does not match the pack (tile_ic=%d, oc_per_wave=%d)",
+                t.tile_ic, t.oc_per_wave, p->tile_ic, p->g);
+  Plan plan;
+  int rc = make_geom(p, N, H, W, stride, pad, t, &plan.geom);
+  if (rc) return rc;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+    return fail(TETRIS_EINVAL, "the first launch of a shape allocates: call tetris_g950_prepare before capturing");
+  rc = g950_bind(p, plan.geom, stream, &plan.entries);
+  if (rc) return rc;
+  memcpy(plan.key, key, sizeof key);
+  std::lock_guard<std::mutex> lock(p->mu);
+  if (p->plans.size() >= 64) p->plans.erase(p->plans.begin());
+  p->plans.push_back(plan);
+  *out = plan;
+  return TETRIS_OK;
+}
+
+size_t partial_bytes_of(const Geom& g) {
+  return g.csplit > 1 ? sizeof(float) * (size_t)g.csplit * g.N * g.K * g.OH * g.OW : 0;
+}
+
+// Partial-sum buffer of a split layer: one per (pack, stream), so that launches of one pack on different streams do
+// not share it.  A buffer that has to grow is replaced, and the old one is kept until the pack is destroyed: a HIP
+// graph captured earlier may still hold its address.
+int partial_buffer(tetris_g950* p, hipStream_t stream, size_t need, bool grow, float** out) {
+  std::lock_guard<std::mutex> lock(p->mu);
+  tetris_g950::Partial& b = p->partial[stream];
+  if (b.bytes < need) {
+    if (!grow)
+      return fail(TETRIS_ENOTFOUND, "no partial-sum buffer of %zu bytes on this stream: call tetris_g950_prepare first",
+                  need);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(TETRIS_EINVAL, "this launch would allocate its partial-sum buffer: call tetris_g950_prepare before "
+                  "capturing");
+    float* d = nullptr;
+    TETRIS_HIP(hipMalloc(&d, need));
+    if (b.ptr) p->retired.push_back(b.ptr);
+    b.ptr = d;
+    b.bytes = need;
+  }
+  *out = b.ptr;
+  return TETRIS_OK;
+}
+
+int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
+               const tetris_tile* tile, hipStream_t stream) {
+  if (!p || !d_in || !d_out) return fail(TETRIS_EINVAL, "null argument");
+  Plan plan;
+  int rc = find_plan(p, N, H, W, stride, pad, tile, stream, true, &plan);
+  if (rc) return rc;
   float* d_partial = nullptr;
   if (plan.geom.csplit > 1) {
-    const Geom& g = plan.geom;
-    const size_t need = sizeof(float) * (size_t)g.csplit * g.N * g.K * g.OH * g.OW;
-    std::lock_guard<std::mutex> lock(p->mu);
-    if (p->partial_bytes < need) {
-      if (p->d_partial) TETRIS_HIP(hipFree(p->d_partial));  // waits for launches that still use it
-      p->d_partial = nullptr;
-      p->partial_bytes = 0;
-      TETRIS_HIP(hipMalloc(&p->d_partial, need));
-      p->partial_bytes = need;
-    }
-    d_partial = p->d_partial;
+    rc = partial_buffer(p, stream, partial_bytes_of(plan.geom), true, &d_partial);
+    if (rc) return rc;
   }
   return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, p->d_grp_off, p->d_oc_order, stream);
 }
@@ -98,25 +131,37 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
 int time_launches(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
                   const tetris_tile* tile, hipStream_t stream, int warm, int repeat, float* ms_out) {
   if (repeat <= 0 || warm < 0) return fail(TETRIS_EINVAL, "bad warm/repeat");
-  hipEvent_t a, b;
-  TETRIS_HIP(hipEventCreate(&a));
-  TETRIS_HIP(hipEventCreate(&b));
-  int rc = TETRIS_OK;
-  for (int i = 0; i < warm && rc == TETRIS_OK; ++i) rc = run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, stream);
-  if (rc == TETRIS_OK) {
-    TETRIS_HIP(hipStreamSynchronize(stream));
-    TETRIS_HIP(hipEventRecord(a, stream));
-    for (int i = 0; i < repeat && rc == TETRIS_OK; ++i)
-      rc = run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, stream);
-    TETRIS_HIP(hipEventRecord(b, stream));
-    TETRIS_HIP(hipEventSynchronize(b));
-    float ms = 0;
-    TETRIS_HIP(hipEventElapsedTime(&ms, a, b));
-    if (ms_out) *ms_out = ms / repeat;
+  hipEvent_t a = nullptr, b = nullptr;
+  auto done = [&](int code) {
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+    return code;
+  };
+#define HIPT(call)                                                                                          \
+  do {                                                                                                      \
+    hipError_t e_ = (call);                                                                                 \
+    if (e_ != hipSuccess)                                                                                   \
+      return done(fail(TETRIS_EHIP, "%s failed at %s:%d: %s", #call, __FILE__, __LINE__, hipGetErrorString(e_))); \
+  } while (0)
+  HIPT(hipEventCreate(&a));
+  HIPT(hipEventCreate(&b));
+  for (int i = 0; i < warm; ++i) {
+    const int rc = run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, stream);
+    if (rc) return done(rc);
   }
-  (void)hipEventDestroy(a);
-  (void)hipEventDestroy(b);
-  return rc;
+  HIPT(hipStreamSynchronize(stream));
+  HIPT(hipEventRecord(a, stream));
+  for (int i = 0; i < repeat; ++i) {
+    const int rc = run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, stream);
+    if (rc) return done(rc);
+  }
+  HIPT(hipEventRecord(b, stream));
+  HIPT(hipEventSynchronize(b));
+  float ms = 0;
+  HIPT(hipEventElapsedTime(&ms, a, b));
+#undef HIPT
+  if (ms_out) *ms_out = ms / repeat;
+  return done(TETRIS_OK);
 }
 
 // Shared body of the two host-to-host entry points.
@@ -372,6 +417,20 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
                            const tetris_tile* tile, void* stream) {
   return run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, static_cast<hipStream_t>(stream));
+}
+
+int tetris_g950_prepare(tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile* tile, void* stream_) {
+  if (!p) return fail(TETRIS_EINVAL, "null argument");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  Plan plan;
+  int rc = find_plan(p, N, H, W, stride, pad, tile, stream, true, &plan);
+  if (rc) return rc;
+  if (plan.geom.csplit > 1) {
+    float* d_partial = nullptr;
+    rc = partial_buffer(p, stream, partial_bytes_of(plan.geom), true, &d_partial);
+    if (rc) return rc;
+  }
+  return TETRIS_OK;
 }
 
 int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,

@@ -153,9 +153,15 @@ struct tetris_g950 {
   // (LDS byte offset | accumulator index << 16 | 0xC << 28, value) pairs for one tile geometry, made on first use
   std::map<tetris::BoundKey, int2*> bound;
   std::vector<tetris::Plan> plans;  // few per pack; searched linearly, most recent first
-  // partial sums of layers whose channel reduction is split over workgroups: [csplit][N][K][OH][OW], grown on demand
-  float* d_partial = nullptr;
-  size_t partial_bytes = 0;
+  // partial sums of layers whose channel reduction is split over workgroups: [csplit][N][K][OH][OW], one buffer per
+  // stream the pack is launched on, made by tetris_g950_prepare or by the first such launch; a buffer that had to
+  // grow is kept (`retired`) until the pack is destroyed, because a captured graph may still hold its address
+  struct Partial {
+    float* ptr = nullptr;
+    size_t bytes = 0;
+  };
+  std::map<hipStream_t, Partial> partial;
+  std::vector<float*> retired;
   std::mutex mu;
   // host mirrors, filled by tetris_g950_host_arrays
   std::vector<int32_t> h_grp_off, h_grp_nnz, h_position, h_oc_order;

@@ -246,7 +246,8 @@ void tetris_g950_destroy(tetris_g950* p) {
   (void)hipFree(p->d_position);
   (void)hipFree(p->d_values);
   (void)hipFree(p->d_oc_order);
-  (void)hipFree(p->d_partial);
+  for (auto& kv : p->partial) (void)hipFree(kv.second.ptr);
+  for (float* d : p->retired) (void)hipFree(d);
   delete p;
 }
 

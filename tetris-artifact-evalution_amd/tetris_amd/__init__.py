@@ -104,6 +104,7 @@ _lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.PO
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
 _lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile),
                                                                                                 C.c_void_p]
+_lib.tetris_g950_prepare.argtypes = [C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile), C.c_void_p]
 _lib.tetris_spconv2d_launch_spf.argtypes = [C.c_void_p] * 7 + [C.c_int] * 8 + [C.c_void_p]
 _lib.tetris_spconv2d_time.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
     C.POINTER(Tile), C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float)]
@@ -243,6 +244,11 @@ class G950Filter:
         _check(_lib.tetris_spconv2d_launch(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h, img_w,
                                            stride, padding, C.byref(tile) if tile is not None else None,
                                            C.c_void_p(stream)))
+
+    def prepare(self, batch, img_h, img_w, stride, padding, tile=None, stream=0):
+        """Makes the launch plan (and a split layer's partial-sum buffer on `stream`) ahead of the first launch."""
+        _check(_lib.tetris_g950_prepare(self._h, batch, img_h, img_w, stride, padding,
+                                        C.byref(tile) if tile is not None else None, C.c_void_p(stream)))
 
     def time(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0, warm=30, repeat=100):
         ms = C.c_float()
