@@ -22,7 +22,7 @@ enum {
   TETRIS_EINVAL = 1,      /* bad argument (shape, NULL, ks > 7, ...) */
   TETRIS_EHIP = 2,        /* a HIP call failed */
   TETRIS_EUNSUPPORTED = 3,/* reference behaviour undefined for this input (see tetris_spf_create) */
-  TETRIS_ENOTFOUND = 4,   /* raw device arrays not produced by a live tetris_spf handle */
+  TETRIS_ENOTFOUND = 4,   /* raw device arrays not produced by a live tetris_spf handle; or no launch plan prepared */
   TETRIS_EIO = 5          /* weight file cannot be opened or is truncated */
 };
 
@@ -178,6 +178,22 @@ int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output
  * (Tetris/spconv2d_utils.h:248-264) before the launcher runs. */
 int tetris_g950_prepare(tetris_g950* p, int batch, int img_h, int img_w, int stride, int padding,
                         const tetris_tile* tile, void* stream);
+
+/* tetris_spconv2d_launch for callers that cannot allocate device memory (code under HIP graph capture, serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It allocates nothing: the launch plan
+ * must exist already (tetris_g950_prepare or an earlier tetris_spconv2d_launch with the same shape and tile, else
+ * TETRIS_ENOTFOUND), and the partial sums of a split layer go to a static device array of
+ * TETRIS_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.  A layer whose
+ * partial sums need more is refused with TETRIS_EINVAL.  All calls on one GPU share that array: calls that overlap in
+ * time on one GPU (different streams or threads) race; calls on one stream are ordered by the stream.  Results are
+ * bit-identical to tetris_spconv2d_launch's. */
+#define TETRIS_NOALLOC_SCRATCH_BYTES (64u << 20)
+int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h,
+                                   int img_w, int stride, int padding, const tetris_tile* tile, void* stream);
+size_t tetris_noalloc_scratch_bytes(void); /* bytes of the array the entry point may use right now */
+/* Lets the entry point use only the first `bytes` of the array (0 or more than TETRIS_NOALLOC_SCRATCH_BYTES = all of
+ * it); returns the limit now in force.  For harnesses that want a larger layer refused rather than run. */
+size_t tetris_noalloc_scratch_limit(size_t bytes);
 
 /* Same call shape as the reference launcher: the raw device arrays of a live tetris_spf (looked up by
  * `d_values`).  tile_h/tile_w are accepted for source compatibility and ignored. */

@@ -7,6 +7,7 @@
 #include <fstream>
 
 #include <algorithm>
+#include <atomic>
 
 #include "common.h"
 
@@ -126,6 +127,32 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
     if (rc) return rc;
   }
   return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, p->d_grp_off, p->d_oc_order, stream);
+}
+
+// ---- scratch of the entry point that allocates nothing ------------------------------------------------------------
+// Partial sums of split layers for callers that cannot allocate.  One array per GPU, held until the process ends;
+// every call on a GPU shares it, so calls that overlap in time on one GPU race.
+constexpr size_t kStaticScratchBytes = (size_t)TETRIS_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) __attribute__((used)) float scratch[kStaticScratchBytes / sizeof(float)];
+
+std::atomic<size_t> g_scratch_limit{kStaticScratchBytes};  // bytes of the array the entry point may use
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, looked up once per device
+
+int static_scratch(float** out) {
+  int dev = -1;
+  TETRIS_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(TETRIS_EINVAL, "device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    TETRIS_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(TETRIS_EHIP, "hipGetSymbolAddress returned a null address for the scratch array");
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return TETRIS_OK;
 }
 
 int time_launches(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
@@ -430,7 +457,38 @@ int tetris_g950_prepare(tetris_g950* p, int N, int H, int W, int stride, int pad
     rc = partial_buffer(p, stream, partial_bytes_of(plan.geom), true, &d_partial);
     if (rc) return rc;
   }
-  return TETRIS_OK;
+  float* s = nullptr;
+  return static_scratch(&s);  // looks the static scratch array of this GPU up, for tetris_spconv2d_launch_noalloc
+}
+
+size_t tetris_noalloc_scratch_bytes(void) { return g_scratch_limit.load(); }
+
+size_t tetris_noalloc_scratch_limit(size_t bytes) {
+  if (bytes == 0 || bytes > kStaticScratchBytes) bytes = kStaticScratchBytes;
+  g_scratch_limit.store(bytes);
+  return bytes;
+}
+
+int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride,
+                                   int pad, const tetris_tile* tile, void* stream_) {
+  if (!p || !d_in || !d_out) return fail(TETRIS_EINVAL, "null argument");
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  Plan plan;
+  int rc = find_plan(p, N, H, W, stride, pad, tile, stream, false, &plan);
+  if (rc) return rc;
+  float* d_partial = nullptr;
+  if (plan.geom.csplit > 1) {
+    const size_t need = partial_bytes_of(plan.geom);
+    const size_t limit = g_scratch_limit.load();
+    if (need > limit)
+      return fail(TETRIS_EINVAL, "this layer needs %zu bytes of partial sums, the static scratch holds %zu: use "
+                  "tetris_spconv2d_launch", need, limit);
+    rc = static_scratch(&d_partial);
+    if (rc) return rc;
+  }
+  // Every element of the partial sums that reduce_kernel reads is written by this launch's conv kernel first, so
+  // what an earlier call left in the array needs no clearing.
+  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, p->d_grp_off, p->d_oc_order, stream);
 }
 
 int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,

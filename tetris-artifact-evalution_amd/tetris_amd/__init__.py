@@ -105,6 +105,10 @@ _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.PO
 _lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile),
                                                                                                 C.c_void_p]
 _lib.tetris_g950_prepare.argtypes = [C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile), C.c_void_p]
+_lib.tetris_spconv2d_launch_noalloc.argtypes = _lib.tetris_spconv2d_launch.argtypes
+_lib.tetris_noalloc_scratch_bytes.restype = C.c_size_t
+_lib.tetris_noalloc_scratch_limit.argtypes = [C.c_size_t]
+_lib.tetris_noalloc_scratch_limit.restype = C.c_size_t
 _lib.tetris_spconv2d_launch_spf.argtypes = [C.c_void_p] * 7 + [C.c_int] * 8 + [C.c_void_p]
 _lib.tetris_spconv2d_time.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
     C.POINTER(Tile), C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float)]
@@ -250,6 +254,12 @@ class G950Filter:
         _check(_lib.tetris_g950_prepare(self._h, batch, img_h, img_w, stride, padding,
                                         C.byref(tile) if tile is not None else None, C.c_void_p(stream)))
 
+    def launch_noalloc(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0):
+        """launch() for callers that cannot allocate: needs prepare() first, uses the library's static scratch array."""
+        _check(_lib.tetris_spconv2d_launch_noalloc(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h,
+                                                   img_w, stride, padding, C.byref(tile) if tile is not None else None,
+                                                   C.c_void_p(stream)))
+
     def time(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0, warm=30, repeat=100):
         ms = C.c_float()
         _check(_lib.tetris_spconv2d_time(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h, img_w,
@@ -270,6 +280,16 @@ def tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, strid
     _check(_lib.tetris_tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
                                    C.byref(t)))
     return t
+
+
+def noalloc_scratch_bytes():
+    """Size of the static device array launch_noalloc keeps the partial sums of split layers in."""
+    return int(_lib.tetris_noalloc_scratch_bytes())
+
+
+def noalloc_scratch_limit(nbytes):
+    """Restricts launch_noalloc to the first `nbytes` of its array (0 = all of it); -> the limit in force."""
+    return int(_lib.tetris_noalloc_scratch_limit(nbytes))
 
 
 def tile_table_load(path):
