@@ -111,6 +111,44 @@ def test_every_tile_shape(env, tile, conv):
         assert ran >= 1, (tile, conv)
 
 
+FLAT_TILES = [  # quads, oc_per_wave, waves: the flat (lanes_w = 64) tiles of pointwise layers
+    (1, 8, 16), (1, 2, 16), (1, 1, 16), (2, 8, 16), (2, 4, 16), (2, 1, 16), (2, 16, 8), (4, 8, 8), (1, 8, 8),
+    (2, 8, 8), (1, 16, 8), (1, 4, 8), (2, 2, 8)]
+
+
+@pytest.mark.parametrize("tile", FLAT_TILES)
+@pytest.mark.parametrize("shape", [(3, 12, 23, 29, 37), (5, 70, 7, 7, 130), (2, 33, 13, 13, 16), (1, 8, 20, 12, 260),
+                                   (17, 5, 3, 3, 40), (2, 300, 14, 14, 24)])
+def test_flat_tiles_of_pointwise_layers(env, tile, shape):
+    # 1x1, stride 1, no padding: a lane owns four consecutive pixels of an image.  Shapes with H*W not a multiple of
+    # four (short last quad, unaligned 16-byte loads, dword stores), ragged channel counts, more images than a unit
+    # holds, and enough input channels for the reduction to be split over workgroups.
+    T, torch, O = env
+    nq, g, waves = tile
+    N, C, H, W, K = shape
+    rng = np.random.default_rng(nq * 100 + g * 10 + waves + C)
+    w = sparse_filter(rng, K, C, 1, 0.7)
+    x = relu_like(rng, (N, C, H, W)) + 0.25
+    ref = O.host_conv2d(x.astype(np.float32), w, 1, 0, threads=4)
+    ran = 0
+    for tile_ic in (1, 5, 16, 64):
+        t = T.Tile(64, nq, g, waves, tile_ic)
+        pk = T.G950Filter(w, tile_ic, g)
+        try:
+            y = run_conv(T, torch, pk, x.astype(np.float32), K, 1, 1, 0, t)
+        except T.TetrisError as e:
+            assert e.code == T.EINVAL and "LDS" in str(e), str(e)
+            continue
+        ran += 1
+        assert max_rel_err(y, ref) <= TOL, (tile, shape, tile_ic)
+    assert ran >= 3
+    # flat tiles are for pointwise layers only
+    with pytest.raises(T.TetrisError) as e:
+        run_conv(T, torch, T.G950Filter(sparse_filter(rng, K, C, 3, 0.7), 8, g), x.astype(np.float32), K, 3, 1, 1,
+                 T.Tile(64, nq, g, waves, 8))
+    assert e.value.code == T.EINVAL
+
+
 def test_channel_order_is_honoured(env):
     T, torch, O = env
     N, C, H, W, K, ks = 2, 16, 11, 11, 72, 3

@@ -374,7 +374,8 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
   std::vector<tetris_tile> ranked;
   int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked);
   if (rc) return rc;
-  if (max_candidates <= 0) max_candidates = 24;
+  if (max_candidates == 0) max_candidates = 24;
+  if (max_candidates < 0) max_candidates = (int)ranked.size();  // exhaustive, like the reference's table walk
   const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
   const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
   const size_t f_bytes = sizeof(float) * (size_t)C * K * ks * ks;

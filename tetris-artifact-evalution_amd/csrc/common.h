@@ -36,11 +36,14 @@ constexpr int kTileBytes = 65536;  // LDS bytes of one workgroup's input tile (a
 constexpr int kBufBytes = 54272;   // one LDS buffer of the triple-buffered kernel (8-wave workgroups, 3 * 53 KiB)
 constexpr int kHalfBufBytes = 27136;  // ... when two 8-wave workgroups of 64-accumulator waves share a CU
 constexpr int kBufs = 3;
+constexpr int kFlatBufBytes = 65536;      // one of the two LDS buffers of a flat (pointwise) kernel, one workgroup per CU
+constexpr int kFlatHalfBufBytes = 32768;  // ... of its 8-wave form with 64 accumulators, two workgroups per CU
 constexpr int kMaxChunks = 8;      // (6 in a 16-wave workgroup, whose waves have fewer registers)
 constexpr int kMaxChunks16 = 6;
 //      // 64-dword LDS chunks of one staged channel a wave may own (triple-buffered kernel)
 constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4 * quads
 constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
+constexpr int kFlatLanes = 64;   // tetris_tile.lanes_w of the flat (pointwise) tiles
 constexpr int kMaxSplit = 8;      // most workgroups that may share an output tile (each reduces a slice of the stages)
 
 inline int out_extent(int in, int pad, int ks, int stride) { return (in + 2 * pad - ks) / stride + 1; }
@@ -103,6 +106,14 @@ struct Geom {
   // quad j belongs to image j >> jsh of the unit and to column group j & ((1 << jsh) - 1).  fold = 1, jsh = 2 otherwise.
   int fold, jsh;
   int stagers;         // waves 0 .. stagers-1 fill LDS (4 or 8 of an 8-wave workgroup; 4, 8 or 16 of a 16-wave one)
+  // Pointwise layers (1x1, stride 1, no padding; ver == 4): no halo, so the pixels of an image are one flat run of H*W
+  // floats per channel and a lane owns four CONSECUTIVE pixels (a quad).  Image n holds `qi` = ceil(H*W / 4) quads,
+  // the batch N*qi quads, a unit 64 consecutive quads of that sequence (lane l of unit u: quad u*64 + l), and LDS one
+  // 1 KiB row per staged channel and unit (lane l at byte 16*l): staging is one 16-byte-per-lane load that writes LDS
+  // directly per (channel, unit), reads are aligned 16-byte accesses at consecutive addresses, stores are 16 bytes
+  // per lane when H*W is a multiple of four.
+  int qi, quads_total;
+  unsigned m_qi;
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan

@@ -21,7 +21,8 @@ Variants (macro suffix): ""  one 64 KiB LDS tile, 128 accumulators, 16-bit LDS a
                          "3" three LDS buffers (addresses up to 160 KiB), 128 accumulators;
                          "4" three LDS buffers, 64 accumulators and at most 64 VGPRs below them, so that four
                              waves fit a SIMD (measured: 56 TFLOP/s for the loop alone against 43-50 with two);
-                         "5" as "4" with buffers of half the size, for two 8-wave workgroups per CU.
+                         "5" as "4" with buffers of half the size, for two 8-wave workgroups per CU;
+                         "6", "7", "8" as "4", "3", "5" for the flat kernels' LDS buffers of 64 / 64 / 32 KiB.
 
 Per entry the loop issues: NQ ds_read_b128, one s_lshr (M0), one s_waitcnt, 4*NQ v_fma; per batch: one
 s_load_dwordx16, eight v_add_u16 (addresses), a handful of scalar ops.
@@ -30,6 +31,8 @@ s_load_dwordx16, eight v_add_u16 (addresses), a handful of scalar ops.
 TILE_BYTES = 65536   # LDS tile of the single-buffered kernel
 BUF_BYTES = 54272    # one of the three LDS buffers of the triple-buffered kernels (3 * 53 KiB <= 160 KiB)
 HALF_BUF_BYTES = 27136  # ... when two workgroups share a CU
+FLAT_BUF_BYTES = 65536       # one of the two LDS buffers of the flat (pointwise) kernels
+FLAT_HALF_BUF_BYTES = 32768  # ... when two workgroups share a CU
 
 # record sizes to emit loops for; the pack only makes single-entry records so far (2 and 4 measured 1.1-1.2x)
 SHARES = (1,)
@@ -39,6 +42,10 @@ VARIANTS = {
     "3": dict(wide=True, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}),
     "4": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}),
     "5": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}, buf=HALF_BUF_BYTES),
+    # flat tiles of pointwise layers: two LDS buffers of 64 KiB (one workgroup per CU) or 32 KiB (two per CU)
+    "6": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}, buf=FLAT_BUF_BYTES),
+    "7": dict(wide=True, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}, buf=FLAT_BUF_BYTES),
+    "8": dict(wide=True, acc0=64, nacc=64, nbuf={1: 4, 2: 2}, buf=FLAT_HALF_BUF_BYTES),
 }
 
 
@@ -168,6 +175,8 @@ def main():
     print("#define TETRIS_WALK_TILE_BYTES %d" % TILE_BYTES)
     print("#define TETRIS_WALK_BUF_BYTES %d" % BUF_BYTES)
     print("#define TETRIS_WALK_HALF_BUF_BYTES %d" % HALF_BUF_BYTES)
+    print("#define TETRIS_WALK_FLAT_BUF_BYTES %d" % FLAT_BUF_BYTES)
+    print("#define TETRIS_WALK_FLAT_HALF_BUF_BYTES %d" % FLAT_HALF_BUF_BYTES)
 
 
 if __name__ == "__main__":

@@ -123,8 +123,8 @@ int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, int G,
   if (!d_filter || !out) return fail(TETRIS_EINVAL, "null argument");
   if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || tile_ic <= 0)
     return fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d tile_ic=%d (ks <= %d)", C, K, ks, tile_ic, kMaxKs);
-  if (G != 4 && G != 8 && G != 16 && G != 32)
-    return fail(TETRIS_EINVAL, "oc_per_wave must be 4, 8, 16 or 32 (got %d)", G);
+  if (G != 1 && G != 2 && G != 4 && G != 8 && G != 16 && G != 32)
+    return fail(TETRIS_EINVAL, "oc_per_wave must be 1, 2, 4, 8, 16 or 32 (got %d)", G);
   if ((long long)tile_ic * 64 >= (1 << 24))
     return fail(TETRIS_EINVAL, "tile_ic %d does not fit the position word", tile_ic);
   tetris_g950* p = new tetris_g950;

@@ -69,6 +69,61 @@ int image_stride(const Shape& s, int tile_ic, int stride) {
 
 }  // namespace
 
+// Geometry of a flat tile (lanes_w == 64) for a pointwise layer; `g` holds the layer and the tile's quads, slots and waves.
+static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Geom* out) {
+  if (p->ks != 1 || g.stride != 1 || g.pad != 0 || g.step != 1)
+    return fail(TETRIS_EINVAL, "flat tiles (lanes_w = %d) are for 1x1 layers of stride 1 without padding", kFlatLanes);
+  if (t.waves != 8 && t.waves != 16) return fail(TETRIS_EINVAL, "bad tile: flat tiles take 8 or 16 waves (got %d)", t.waves);
+  if (g.nq != 1 && g.nq != 2 && g.nq != 4) return fail(TETRIS_EINVAL, "bad tile: quads=%d", g.nq);
+  if (t.oc_per_wave != p->g)
+    return fail(TETRIS_EINVAL, "tile wants %d output channels per wave, the pack was made for %d", t.oc_per_wave, p->g);
+  const int acc_regs = t.waves == 16 ? kAccRegs / 2 : kAccRegs;
+  if (g.g * 4 * g.nq > acc_regs || (t.waves == 16 && g.nq > 2))
+    return fail(TETRIS_EINVAL, "oc_per_wave * 4 * quads = %d exceeds the %d accumulators of a wave", g.g * 4 * g.nq, acc_regs);
+  g.ver = 4;
+  const long long hw = (long long)g.H * g.W;
+  g.qi = (int)((hw + 3) / 4);
+  const long long quads = (long long)g.N * g.qi;
+  if (quads * g.qi >= (1ll << 32) || quads >= (1ll << 30))
+    return fail(TETRIS_EINVAL, "too many pixels for the kernel's index arithmetic");
+  g.quads_total = (int)quads;
+  g.m_qi = magic_reciprocal(g.qi);
+  g.buf_bytes = (t.waves == 8 && g.g * 4 * g.nq <= kAccRegs / 2 && g.nq <= 2) ? kFlatHalfBufBytes : kFlatBufBytes;
+  g.region = g.buf_bytes / g.nq;
+  g.plane = 256; g.pitch = 0; g.par = 0; g.lw = g.lr = 64; g.lh = 1; g.thi = 1; g.nb = 1; g.ng = 64; g.ih = 1;
+  g.img_stride = g.tile_ic * g.plane;
+  g.fold = 1; g.jsh = 2;
+  if (4ll * g.img_stride > g.region)
+    return fail(TETRIS_EINVAL, "a pixel unit needs %lld bytes of LDS for %d staged channels (region is %d): lower tile_ic "
+                "or quads", 4ll * g.img_stride, g.tile_ic, g.region);
+  g.units = (int)((quads + 63) / 64);
+  g.units_w = g.units; g.units_h = 1; g.units_n = 1;
+  g.ugroups = ceil_div(g.units, g.nq);
+  g.kb = t.waves * g.g;
+  g.kblocks = ceil_div(p->K, g.kb);
+  if (g.kblocks * g.kb > p->slots) return fail(TETRIS_EINVAL, "channel block %d does not divide the slot padding", g.kb);
+  if ((long long)g.ugroups * g.kblocks > (1ll << 28)) return fail(TETRIS_EINVAL, "grid too large");
+  // a workgroup reaches its images through one 2 GB window on the input and one on the output
+  const long long span = (64ll * g.nq + g.qi - 1) / g.qi + 2;  // images a workgroup's quads can touch, and a spare
+  if (4ll * hw * std::max(p->C, p->K) * span >= (1ll << 31))
+    return fail(TETRIS_EINVAL, "images too large for the 2 GB window of a workgroup");
+  if ((long long)g.N * p->K * hw >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
+  const bool four = t.waves == 16 || g.buf_bytes == kFlatHalfBufBytes;
+  const long long room = 256ll * (four ? 16 : 8);
+  const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
+  g.csplit = 1;
+  while (g.csplit < kMaxSplit && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
+  if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32) ||
+      (long long)g.stages * (g.csplit + 1) * g.csplit >= (1ll << 32))
+    return fail(TETRIS_EINVAL, "grid too large");
+  g.m_kblocks = magic_reciprocal(g.kblocks);
+  g.m_csplit = magic_reciprocal(g.csplit);
+  g.stagers = t.waves;
+  g.spt = 1; g.cg = 1; g.fill_iters = 1;
+  *out = g;
+  return TETRIS_OK;
+}
+
 int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile& t, Geom* out) {
   Geom g{};
   if (N <= 0 || H <= 0 || W <= 0 || stride <= 0 || pad < 0)
@@ -92,6 +147,7 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
   g.nq = t.quads;
   g.g = p->g;
   g.waves = t.waves;
+  if (t.lanes_w == kFlatLanes) return make_flat_geom(p, g, t, out);
   if (t.lanes_w < 1 || t.lanes_w > 64 || (g.nq != 1 && g.nq != 2 && g.nq != 4))
     return fail(TETRIS_EINVAL, "bad tile: lanes_w=%d quads=%d", t.lanes_w, g.nq);
   if (t.oc_per_wave != p->g)
@@ -234,6 +290,7 @@ static int max_tile_ic(const Shape& s, int nq, int g, int waves, int stride, int
 int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad layer shape");
+  const bool pointwise = ks == 1 && stride == 1 && pad == 0;  // what the flat tiles take
   if (ks == 1 && stride > 1 && pad == 0) {  // run as a stride-1 layer on the sub-grid it reads (see make_geom)
     H = (H - 1) / stride + 1;
     W = (W - 1) / stride + 1;
@@ -290,6 +347,38 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
         }
       }
     }
+  }
+  if (pointwise) {
+    // Flat tiles of pointwise layers (lanes_w = 64): a unit is 64 consecutive 4-pixel quads of the batch, two LDS
+    // buffers of 64 KiB (32 KiB for 8 waves of at most 64 accumulators, two workgroups per CU), 1 KiB per staged
+    // channel and unit.  A stage is one walk and one barrier; a walk call costs about 600 cycles before its first entry.
+    static const int kFlatG[] = {32, 16, 8, 4, 2, 1};
+    const long long quads = (long long)N * ((H * W + 3) / 4);
+    for (int waves : {16, 8})
+      for (int nq : {1, 2, 4})
+        for (int g : kFlatG) {
+          const int acc = g * 4 * nq;
+          if (acc > (waves == 16 ? kAccRegs / 2 : kAccRegs) || (waves == 16 && nq > 2) || waves * g > kSlotPad) continue;
+          const bool half = waves == 8 && acc <= kAccRegs / 2 && nq <= 2;
+          const int buf = half ? kFlatHalfBufBytes : kFlatBufBytes;
+          for (int tic = 64; tic >= 8; tic /= 2) {
+            const int t = std::min(tic, C);
+            if (1024 * t * nq > buf) continue;
+            const bool four = waves == 16 || half;
+            const long long ugroups = ((quads + 63) / 64 + nq - 1) / nq;
+            const int kblocks = ceil_div(K, waves * g);
+            const int stages = ceil_div(C, t);
+            const double entries = std::ceil((g * t * density + 0.5) / 8.0) * 8.0;
+            const double per_entry = four ? 40.0 + 70.0 * nq : 35.0 + 41.0 * nq;
+            const double per_wave = stages * (entries * per_entry + 600.0 + 900.0) + 6000.0;
+            const double rounds = (double)ugroups * kblocks * waves / (256.0 * (four ? 16.0 : 8.0));
+            const double cost = per_wave * std::max(rounds, 0.62) * (1.0 + 0.02 * kblocks);
+            tetris_tile tt{};
+            tt.lanes_w = kFlatLanes; tt.quads = nq; tt.oc_per_wave = g; tt.waves = waves; tt.tile_ic = t;
+            scored.emplace_back(cost, tt);
+            if (t == C) break;
+          }
+        }
   }
   if (scored.empty()) return fail(TETRIS_EINVAL, "no tile shape fits this layer");
   std::stable_sort(scored.begin(), scored.end(),
