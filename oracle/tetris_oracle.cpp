@@ -10,9 +10,14 @@
 //                              and the reference's own tensor_utils.cc compiled unmodified
 //                              (oracle/_ref, when the reference checkout is present)
 //   orc_read_weight_file       the compiled reference reader (oracle/_ref) on shipped weight files
-//   orc_spf_pack               FNV-1a known answers of all five arrays recorded from the compiled
-//                              reference for six shipped layers x {plain, BANK_OPTIMIZE +
-//                              REORDER_OUT_CHANNEL} x TILE_IC {32,128}; structural invariants
+//   orc_spf_pack               plain step 1: the scan order the text fixes, invariants, decode == filter non-zeros;
+//                              Bank-SR and ReorderOutChannel: hand-worked cases derived step by step from the text
+//                              of spconv2d_utils.h:99-199 and :275-420 (broadcast pass, free-bank pass, wait-list
+//                              pads, the entry-index-as-bank comparison of :184, cost function with duplicates and
+//                              padding term, ties, two stages, K % 8 != 0), per-step invariants on random filters,
+//                              and both-flags == Bank-SR on the permuted filter (tests/test_oracle_handworked.py);
+//                              as a cross-check, FNV-1a answers recorded from a compiled reference for six shipped
+//                              layers (tests/golden/spf_known_answers.json)
 //   orc_host_spconv2d*,        decode(pack(filter)) convolved == orc_host_conv2d
 //   orc_g950_*                 layout defined by this project (no reference counterpart); pinned by
 //                              multiset equality with the filter's non-zeros and by conv equality
