@@ -127,6 +127,15 @@ int tetris_tile_select(int batch, int img_h, int img_w, int in_channel, int out_
  * Process-wide; may be called several times (later files win). */
 int tetris_tile_table_load(const char* path, int* rows_out);
 
+/* Switches for ablation runs, the counterpart of the reference's build variants (-DBANK_OPTIMIZE / -DREORDER_OUT_CHANNEL
+ * and its ablation binaries, evalution/script/build_ablation.sh:12-18, Tetris/ablation_kernel.cu).  Process-wide; they
+ * act on launch plans made afterwards (a pack keeps the plans it already has).  The initial value is taken from the
+ * environment variable TETRIS_OPTIONS (a number) when it is set, else 0. */
+#define TETRIS_OPT_PAIRS 1u        /* halo'd kernels walk streams rearranged into pairs of entries that share one LDS read, then singles */
+#define TETRIS_OPT_NO_BANK_RULE 2u /* LDS rows packed densely: the lane-row pitch rule that keeps 16-byte LDS reads conflict-free is off */
+int tetris_options_set(unsigned flags);
+unsigned tetris_options_get(void);
+
 /* What this GPU delivers to a plain device copy (GB/s, read + write bytes of a 256 MiB buffer) and to a loop of
  * independent fp32 FMAs (TFLOP/s, non-packed), for reading roofline fractions against measured ceilings as well
  * as nominal ones.  No reference counterpart (the reference prints milliseconds and "T" per layer only,

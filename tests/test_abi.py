@@ -88,7 +88,9 @@ def test_tile_select_is_sane():
     for shape in [(1, 56, 56, 64, 128, 3, 1, 1), (16, 224, 224, 3, 64, 3, 1, 1), (16, 7, 7, 1024, 1024, 1, 1, 0),
                   (4, 224, 224, 3, 64, 7, 2, 3), (16, 13, 13, 1024, 255, 1, 1, 0), (1, 14, 14, 512, 512, 3, 1, 1)]:
         t = T.tile_select(*shape)
-        assert 1 <= t.lanes_w <= 62 and t.quads in (1, 2, 4) and t.oc_per_wave in (4, 8, 16, 32)
+        flat = t.lanes_w == 64  # flat tiles: pointwise layers only, 8 or 16 waves
+        assert (1 <= t.lanes_w <= 62 or (flat and shape[5:] == (1, 1, 0) and t.waves in (8, 16)))
+        assert t.quads in (1, 2, 4) and t.oc_per_wave in (1, 2, 4, 8, 16, 32)
         assert t.oc_per_wave * 4 * t.quads <= (64 if t.waves == 16 else 128) and t.waves in (1, 2, 4, 8, 16) and t.tile_ic >= 1
     with pytest.raises(T.TetrisError):
         T.tile_select(0, 5, 5, 3, 3, 3, 1, 1)

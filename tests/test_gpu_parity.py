@@ -149,6 +149,37 @@ def test_flat_tiles_of_pointwise_layers(env, tile, shape):
     assert e.value.code == T.EINVAL
 
 
+@pytest.mark.parametrize("opts", [1, 2, 3])
+def test_ablation_switches_keep_the_results(env, opts):
+    # TETRIS_OPT_PAIRS (streams rearranged into pairs sharing an LDS read + singles) and TETRIS_OPT_NO_BANK_RULE (LDS
+    # rows packed densely, bank conflicts allowed) change how the kernels run, never what they compute.  Channel
+    # orders: file order, the reference's ReorderOutChannel permutation, the balanced order.
+    T, torch, O = env
+    rng = np.random.default_rng(40 + opts)
+    cases = [(3, 40, 23, 29, 64, 3, 1, 1, (14, 2, 8, 16, 8)), (2, 24, 30, 30, 48, 3, 2, 1, (8, 1, 8, 4, 4)),
+             (2, 3, 33, 33, 16, 7, 2, 3, (9, 1, 16, 4, 3)), (4, 96, 14, 14, 128, 1, 1, 0, (14, 1, 8, 4, 32)),
+             (2, 64, 28, 28, 64, 3, 1, 1, (14, 2, 16, 8, 8)), (2, 32, 20, 20, 32, 5, 1, 2, (5, 1, 4, 8, 2))]
+    assert T.options_get() == 0
+    try:
+        T.options_set(opts)
+        assert T.options_get() == opts
+        for N, C, H, W, K, ks, stride, pad, tile in cases:
+            w = sparse_filter(rng, K, C, ks, 0.6)  # dense enough for many entries to share a position
+            x = relu_like(rng, (N, C, H, W))
+            ref = O.host_conv2d(x, w, stride, pad, threads=4)
+            tile = T.Tile(*tile)
+            ref_order = T.SparseFilter(w, C, K, ks, 32, True, True, T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL).oc_permutation_
+            for order in (None, ref_order, "balanced"):
+                pk = T.G950Filter.for_tile(w, tile, oc_order=order)
+                y = run_conv(T, torch, pk, x, K, ks, stride, pad, tile)
+                assert max_rel_err(y, ref) <= TOL, (opts, tile, order is None)
+                pk.close()
+        with pytest.raises(T.TetrisError):
+            T.options_set(0x100)
+    finally:
+        T.options_set(0)
+
+
 def test_channel_order_is_honoured(env):
     T, torch, O = env
     N, C, H, W, K, ks = 2, 16, 11, 11, 72, 3

@@ -77,7 +77,7 @@ int find_plan(tetris_g950* p, int N, int H, int W, int stride, int pad, const te
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
     return fail(TETRIS_EINVAL, "the first launch of a shape allocates: call tetris_g950_prepare before capturing");
-  rc = g950_bind(p, plan.geom, stream, &plan.entries);
+  rc = g950_bind(p, plan.geom, geom_walks_pairs(plan.geom), stream, &plan.entries, &plan.grp_off, &plan.grp_pair);
   if (rc) return rc;
   memcpy(plan.key, key, sizeof key);
   std::lock_guard<std::mutex> lock(p->mu);
@@ -126,7 +126,7 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
     rc = partial_buffer(p, stream, partial_bytes_of(plan.geom), true, &d_partial);
     if (rc) return rc;
   }
-  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, p->d_grp_off, p->d_oc_order, stream);
+  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, stream);
 }
 
 // ---- scratch of the entry point that allocates nothing ------------------------------------------------------------
@@ -351,6 +351,14 @@ int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* o) {
   return TETRIS_OK;
 }
 
+int tetris_options_set(unsigned flags) {
+  if (flags & ~(TETRIS_OPT_PAIRS | TETRIS_OPT_NO_BANK_RULE))
+    return fail(TETRIS_EINVAL, "unknown option bits 0x%x", flags);
+  set_options(flags);
+  return TETRIS_OK;
+}
+unsigned tetris_options_get(void) { return options(); }
+
 int tetris_tile_select(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* out) {
   if (!out) return fail(TETRIS_EINVAL, "null argument");
   return choose_tile(N, H, W, C, K, ks, stride, pad, out);
@@ -489,7 +497,7 @@ int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_in, float* d_o
   }
   // Every element of the partial sums that reduce_kernel reads is written by this launch's conv kernel first, so
   // what an earlier call left in the array needs no clearing.
-  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, p->d_grp_off, p->d_oc_order, stream);
+  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, stream);
 }
 
 int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,

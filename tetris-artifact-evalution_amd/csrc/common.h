@@ -129,7 +129,9 @@ inline int lds_entry_offset(int plane, int pitch, int par, int stride, int ic_lo
 
 struct BoundKey {
   int plane, pitch, par, stride, nq;
+  int paired;  // 1: streams rearranged into a segment of pairs and a segment of singles (see g950_bind)
   bool operator<(const BoundKey& o) const {
+    if (paired != o.paired) return paired < o.paired;
     if (plane != o.plane) return plane < o.plane;
     if (pitch != o.pitch) return pitch < o.pitch;
     if (par != o.par) return par < o.par;
@@ -145,7 +147,9 @@ namespace tetris {
 struct Plan {
   int key[10];  // N, H, W, stride, pad, lanes_w, quads, oc_per_wave, waves, tile_ic
   Geom geom;
-  const int2* entries;
+  const int2* entries;        // the pack's entries bound to the geometry
+  const int32_t* grp_off;     // [groups*stages+1] first entry of every stream in `entries`
+  const int32_t* grp_pair;    // [groups*stages] entries of the stream's leading segment of pairs (0 when unpaired)
 };
 }  // namespace tetris
 
@@ -163,6 +167,13 @@ struct tetris_g950 {
   int32_t* d_oc_order = nullptr;  // [slots], -1 for padding slots
   // (LDS byte offset | accumulator index << 16 | 0xC << 28, value) pairs for one tile geometry, made on first use
   std::map<tetris::BoundKey, int2*> bound;
+  // Paired arrangement of the streams (made on the first paired bind; depends on the pack only): two consecutive
+  // entries of a stream that share their position become a pair; per stream first all pairs, padded to a multiple
+  // of 8 entries, then the entries left single, padded likewise.
+  int32_t* d_pgrp_off = nullptr;   // [groups*stages+1]
+  int32_t* d_pgrp_pair = nullptr;  // [groups*stages]
+  int32_t* d_zero_pair = nullptr;  // [groups*stages] zeros: the pair counts of the unpaired arrangement
+  int64_t n_paired_entries = 0;
   std::vector<tetris::Plan> plans;  // few per pack; searched linearly, most recent first
   // partial sums of layers whose channel reduction is split over workgroups: [csplit][N][K][OH][OW], one buffer per
   // stream the pack is launched on, made by tetris_g950_prepare or by the first such launch; a buffer that had to
@@ -198,9 +209,13 @@ int spf_pack_host(const float* filter, int C, int K, int ks, int tile_ic, bool a
                   unsigned flags, tetris_spf* out);
 
 // spf_pack_device.hip
-int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** entries_out);
+// entries of the pack bound to geometry `g`; paired: rearranged into pairs and singles (kernels that walk pairs)
+int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, const int2** entries_out,
+              const int32_t** grp_off_out, const int32_t** grp_pair_out);
 
 // tile_select.cpp
+unsigned options();  // TETRIS_OPT_* flags in force (tetris_options_set, or the environment variable TETRIS_OPTIONS)
+void set_options(unsigned flags);
 int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile& t, Geom* g);
 int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, tetris_tile* t);
 // reads rows in the format of tuned_tiles.inc; choose_tile looks them up before the built-in table
@@ -215,7 +230,9 @@ int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_til
 // launches the conv; when the geometry splits the channel reduction (csplit > 1) the workgroups write their partial
 // sums to d_partial ([csplit] outputs) and a second kernel adds the slices, in order, into d_out
 int launch_conv(const Geom& g, const float* d_in, float* d_out, float* d_partial, const int2* entries,
-                const int32_t* grp_off, const int32_t* oc_order, hipStream_t stream);
+                const int32_t* grp_off, const int32_t* grp_pair, const int32_t* oc_order, hipStream_t stream);
+// whether the kernel of geometry `g` walks paired streams
+bool geom_walks_pairs(const Geom& g);
 
 }  // namespace tetris
 

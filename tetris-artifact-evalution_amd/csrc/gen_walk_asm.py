@@ -34,8 +34,9 @@ HALF_BUF_BYTES = 27136  # ... when two workgroups share a CU
 FLAT_BUF_BYTES = 65536       # one of the two LDS buffers of the flat (pointwise) kernels
 FLAT_HALF_BUF_BYTES = 32768  # ... when two workgroups share a CU
 
-# record sizes to emit loops for; the pack only makes single-entry records so far (2 and 4 measured 1.1-1.2x)
-SHARES = (1,)
+# record sizes to emit loops for: single entries, and pairs of entries that share one set of LDS reads (the same input
+# position for two output channels of the wave).  The flat kernels' waves hold few channels: singles only.
+SHARES = {"": (1, 2), "3": (1, 2), "4": (1, 2), "5": (1, 2), "6": (1,), "7": (1,), "8": (1,)}
 
 VARIANTS = {
     "": dict(wide=False, acc0=128, nacc=128, nbuf={1: 4, 2: 4, 4: 2}),
@@ -135,6 +136,8 @@ def walk(nq, variant="", share=1):
                 L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
                 if kk == 0:
                     L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
+                else:
+                    L.append("s_nop 0")  # keeps one instruction between the write of M0 and the indexed VALU use
                 L += fmas(c, r % nbuf, 37 + 2 * e)
         for i in range(8):
             L.append("s_mov_b64 s[%d:%d], s[%d:%d]" % (36 + 2 * i, 37 + 2 * i, 52 + 2 * i, 53 + 2 * i))
@@ -163,7 +166,7 @@ def main():
     print("// Generated by gen_walk_asm.py -- do not edit.")
     for variant, v in VARIANTS.items():
         for nq in sorted(v["nbuf"]):
-            for share in SHARES:
+            for share in SHARES[variant]:
                 c, L = walk(nq, variant, share)
                 print("#define TETRIS_WALK%s_ASM_%d_S%d \\" % (variant, nq, share))
                 for line in L:

@@ -192,24 +192,164 @@ int pack_device(const float* d_filter, int C, int K, int ks, int tile_ic, int G,
 
 }  // namespace
 
-int g950_bind(tetris_g950* p, const Geom& g, hipStream_t stream, const int2** entries_out) {
-  const BoundKey key{g.plane, g.pitch, g.par, g.stride, g.nq};
+namespace {
+
+// Which entries of a stream become pair members.  The stream lists its entries position by position (slots ascending
+// inside a position); of a run of k entries with one position the first 2 * (k / 2) form k / 2 pairs, and the last
+// one of an odd run stays single.  Entry i is therefore single exactly when it is the last of its run and its index
+// inside the run is even.  One wave per stream; returns, per lane, the classification of entry base + lane.
+struct PairScan {
+  int carry_start;  // first entry index of the run that the previous chunk ended in
+  int carry_pos;    // position of the previous chunk's last entry
+};
+
+__device__ __forceinline__ bool entry_is_single(const int32_t* __restrict__ position, int beg, int nnz, int i, int lane,
+                                                PairScan& c) {
+  const int pos = i < nnz ? (position[beg + i] & 0xffffff) : -1;
+  int prev = __shfl_up(pos, 1);
+  if (lane == 0) prev = c.carry_pos;
+  const bool start = i < nnz && (i == 0 || pos != prev);
+  int run_start = start ? i : -1;  // inclusive max-scan over the lanes
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(run_start, off);
+    if (lane >= off) run_start = max(run_start, o);
+  }
+  run_start = max(run_start, c.carry_start);
+  const int next = i + 1 < nnz ? (position[beg + i + 1] & 0xffffff) : -2;
+  const bool last = i < nnz && next != pos;
+  const bool single = last && (((i - run_start) & 1) == 0);
+  c.carry_start = __shfl(run_start, 63);
+  c.carry_pos = __shfl(pos, 63);
+  return single;
+}
+
+__global__ __launch_bounds__(256) void pair_count_kernel(const int32_t* __restrict__ position,
+                                                         const int32_t* __restrict__ grp_off,
+                                                         const int32_t* __restrict__ grp_nnz,
+                                                         int32_t* __restrict__ seg_len, int32_t* __restrict__ seg_pair,
+                                                         int nstream) {
+  const int sid = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (sid >= nstream) return;
+  const int beg = grp_off[sid], nnz = grp_nnz[sid];
+  PairScan c{-1, -3};
+  int singles = 0;
+  for (int i0 = 0; i0 < nnz; i0 += 64) singles += __popcll(__ballot(entry_is_single(position, beg, nnz, i0 + lane, lane, c)));
+  if (lane == 0) {
+    const int pairs = (nnz - singles + kBatch - 1) / kBatch * kBatch;
+    seg_pair[sid] = pairs;
+    seg_len[sid] = pairs + (singles + kBatch - 1) / kBatch * kBatch;
+  }
+}
+
+__global__ __launch_bounds__(256) void bind_pairs_kernel(const int32_t* __restrict__ position,
+                                                         const float* __restrict__ values,
+                                                         const int32_t* __restrict__ grp_off,
+                                                         const int32_t* __restrict__ grp_nnz,
+                                                         const int32_t* __restrict__ pgrp_off,
+                                                         const int32_t* __restrict__ pgrp_pair, int2* __restrict__ out,
+                                                         int nstream, int plane, int pitch, int par, int stride, int nq) {
+  const int sid = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (sid >= nstream) return;
+  const int beg = grp_off[sid], nnz = grp_nnz[sid];
+  const int obeg = pgrp_off[sid], oend = pgrp_off[sid + 1], opair = pgrp_pair[sid];
+  const int2 pad = make_int2((int)0xC0000000u, 0);
+  PairScan c{-1, -3};
+  int np = 0, ns = 0;  // pair members and singles written so far
+  for (int i0 = 0; i0 < nnz; i0 += 64) {
+    const int i = i0 + lane;
+    const bool single = entry_is_single(position, beg, nnz, i, lane, c);
+    const bool live = i < nnz;
+    const unsigned long long ms = __ballot(single), mp = __ballot(live && !single);
+    const unsigned long long below = (1ull << lane) - 1ull;
+    if (live) {
+      const int pos = position[beg + i];
+      const int s = pos & 7, r = (pos >> 3) & 7, ic = (pos >> 6) & 0x3ffff, l = (pos >> 24) & 0xff;
+      int2 e;
+      e.x = 4 * (ic * plane + r * pitch + (s % stride) * par + (s / stride) * 4) | ((l * 4 * nq) << 16) | (int)0xC0000000u;
+      e.y = __float_as_int(values[beg + i]);
+      out[single ? obeg + opair + ns + __popcll(ms & below) : obeg + np + __popcll(mp & below)] = e;
+    }
+    np += __popcll(mp);
+    ns += __popcll(ms);
+  }
+  for (int i = obeg + np + lane; i < obeg + opair; i += 64) out[i] = pad;
+  for (int i = obeg + opair + ns + lane; i < oend; i += 64) out[i] = pad;
+}
+
+__global__ void fill_pad_kernel(int2* __restrict__ out, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = make_int2((int)0xC0000000u, 0);
+}
+
+}  // namespace
+
+int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, const int2** entries_out,
+              const int32_t** grp_off_out, const int32_t** grp_pair_out) {
+  const BoundKey key{g.plane, g.pitch, g.par, g.stride, g.nq, paired ? 1 : 0};
+  const int nseg = p->groups * p->stages;
   std::lock_guard<std::mutex> lock(p->mu);
+  if (!p->d_zero_pair) {
+    TETRIS_HIP(hipMalloc(&p->d_zero_pair, sizeof(int32_t) * std::max(nseg, 1)));
+    TETRIS_HIP(hipMemsetAsync(p->d_zero_pair, 0, sizeof(int32_t) * std::max(nseg, 1), stream));
+  }
+  const int blocks = (nseg + 3) / 4;
+  if (paired && !p->d_pgrp_off) {  // the paired arrangement's stream offsets, once per pack
+    int32_t *d_len = nullptr, *d_off = nullptr, *d_pair = nullptr;
+    auto drop = [&](int rc) {
+      if (d_len) (void)hipFree(d_len);
+      if (rc != TETRIS_OK) {
+        if (d_off) (void)hipFree(d_off);
+        if (d_pair) (void)hipFree(d_pair);
+      }
+      return rc;
+    };
+#define HIPB(call)                                                                                              \
+  do {                                                                                                          \
+    hipError_t e_ = (call);                                                                                     \
+    if (e_ != hipSuccess)                                                                                       \
+      return drop(fail(TETRIS_EHIP, "%s failed at %s:%d: %s", #call, __FILE__, __LINE__, hipGetErrorString(e_))); \
+  } while (0)
+    HIPB(hipMalloc(&d_len, sizeof(int32_t) * nseg));
+    HIPB(hipMalloc(&d_off, sizeof(int32_t) * (nseg + 1)));
+    HIPB(hipMalloc(&d_pair, sizeof(int32_t) * nseg));
+    hipLaunchKernelGGL(pair_count_kernel, dim3(blocks), dim3(256), 0, stream, p->d_position, p->d_grp_off, p->d_grp_nnz,
+                       d_len, d_pair, nseg);
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(1024), 0, stream, d_len, d_off, nseg);
+    HIPB(hipGetLastError());
+    int32_t total = 0;
+    HIPB(hipMemcpyAsync(&total, d_off + nseg, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+    HIPB(hipStreamSynchronize(stream));
+#undef HIPB
+    p->n_paired_entries = total;
+    p->d_pgrp_off = d_off;
+    p->d_pgrp_pair = d_pair;
+    drop(TETRIS_OK);
+  }
   auto it = p->bound.find(key);
   if (it == p->bound.end()) {
     int2* d = nullptr;
-    const long long n = p->n_entries + kBatch;
+    const long long n = (paired ? p->n_paired_entries : p->n_entries) + kBatch;  // a spare batch for the look-ahead fetch
     TETRIS_HIP(hipMalloc(&d, sizeof(int2) * (size_t)n));
-    hipLaunchKernelGGL(bind_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p->d_position, p->d_values,
-                       d, n, g.plane, g.pitch, g.par, g.stride, g.nq);
+    if (paired) {
+      hipLaunchKernelGGL(bind_pairs_kernel, dim3(blocks), dim3(256), 0, stream, p->d_position, p->d_values, p->d_grp_off,
+                         p->d_grp_nnz, p->d_pgrp_off, p->d_pgrp_pair, d, nseg, g.plane, g.pitch, g.par, g.stride, g.nq);
+      hipLaunchKernelGGL(fill_pad_kernel, dim3(1), dim3(64), 0, stream, d + p->n_paired_entries, kBatch);
+    } else {
+      hipLaunchKernelGGL(bind_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p->d_position, p->d_values,
+                         d, n, g.plane, g.pitch, g.par, g.stride, g.nq);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       (void)hipFree(d);
-      return fail(TETRIS_EHIP, "bind_kernel launch failed: %s", hipGetErrorString(e));
+      return fail(TETRIS_EHIP, "bind kernel launch failed: %s", hipGetErrorString(e));
     }
     it = p->bound.emplace(key, d).first;
   }
   *entries_out = it->second;
+  *grp_off_out = paired ? p->d_pgrp_off : p->d_grp_off;
+  *grp_pair_out = paired ? p->d_pgrp_pair : p->d_zero_pair;
   return TETRIS_OK;
 }
 
@@ -246,6 +386,9 @@ void tetris_g950_destroy(tetris_g950* p) {
   (void)hipFree(p->d_position);
   (void)hipFree(p->d_values);
   (void)hipFree(p->d_oc_order);
+  (void)hipFree(p->d_pgrp_off);
+  (void)hipFree(p->d_pgrp_pair);
+  (void)hipFree(p->d_zero_pair);
   for (auto& kv : p->partial) (void)hipFree(kv.second.ptr);
   for (float* d : p->retired) (void)hipFree(d);
   delete p;

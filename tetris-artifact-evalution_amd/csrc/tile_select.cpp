@@ -4,7 +4,9 @@
 // Takes the place of the reference's exhaustive search over 185 compiled {KS, STRIDE, TILE_IC, TILE_H,
 // TILE_W} instantiations (Tetris/spconv2d.cc:90-329, 130 launches and one re-pack per candidate).
 #include <algorithm>
+#include <atomic>
 #include <climits>
+#include <cstdlib>
 #include <cmath>
 #include <cstdio>
 #include <mutex>
@@ -13,6 +15,21 @@
 #include "common.h"
 
 namespace tetris {
+
+namespace {
+std::atomic<unsigned> g_options{~0u};  // ~0: not set yet
+}
+
+unsigned options() {
+  unsigned v = g_options.load();
+  if (v == ~0u) {
+    const char* e = std::getenv("TETRIS_OPTIONS");
+    v = e ? (unsigned)std::strtoul(e, nullptr, 0) & 0xffffu : 0u;
+    g_options.store(v);
+  }
+  return v;
+}
+void set_options(unsigned flags) { g_options.store(flags & 0xffffu); }
 
 namespace {
 
@@ -37,9 +54,10 @@ Shape unit_shape(int lw, int OH, int N, int ks, int stride) {
   double best = 1e300;
   s.lr = lw;
   s.pitch = min_pitch;
+  const bool rule = !(options() & TETRIS_OPT_NO_BANK_RULE);
   for (int lr = lw; lr <= 64 && lr <= lw + 16; ++lr)
     for (int pitch = min_pitch; pitch <= min_pitch + 64; pitch += 4) {
-      if ((stride * pitch - 4 * lr) % bank_period(lr) != 0) continue;
+      if (rule && (stride * pitch - 4 * lr) % bank_period(lr) != 0) continue;
       const int lh = 64 / lr;
       const int thi = std::min(lh, OH);
       const int rows = std::max(1, std::min(lh / thi, N)) * thi;  // lane rows that can hold pixels
@@ -62,7 +80,7 @@ Shape unit_shape(int lw, int OH, int N, int ks, int stride) {
 // row of one image to the first of the next also meets the bank rule.
 int image_stride(const Shape& s, int tile_ic, int stride) {
   int v = tile_ic * s.ih * s.pitch;
-  if (s.nb > 1)
+  if (s.nb > 1 && !(options() & TETRIS_OPT_NO_BANK_RULE))
     while ((v - (s.thi - 1) * stride * s.pitch - 4 * s.lr) % bank_period(s.lr) != 0) v += 4;
   return v;
 }
@@ -580,6 +598,27 @@ int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_til
     for (int w = 0; w < waves; ++w)
       for (int32_t k : members[w]) *o++ = k;
   }
+  // The deal is a heuristic: keep the file order when it is no worse by the measure the deal aims at (what the waves
+  // of a workgroup wait for: per block and stage the busiest wave's entries, summed).
+  auto wait_cost = [&](auto channel_at) {
+    int64_t sum = 0;
+    for (int b = 0; b < nblocks; ++b)
+      for (int s = 0; s < S; ++s) {
+        int64_t worst = 0;
+        for (int w = 0; w < waves; ++w) {
+          int64_t n = 0;
+          for (int i = 0; i < G; ++i) {
+            const int slot = b * B + w * G + i;
+            if (slot < K) n += per[(size_t)channel_at(slot) * S + s];
+          }
+          worst = std::max(worst, n);
+        }
+        sum += worst;
+      }
+    return sum;
+  };
+  if (wait_cost([&](int slot) { return slot; }) <= wait_cost([&](int slot) { return order[slot]; }))
+    for (int k = 0; k < K; ++k) order[k] = k;
   return TETRIS_OK;
 }
 

@@ -46,6 +46,7 @@ BANK_OPTIMIZE = 1
 REORDER_OUT_CHANNEL = 2
 
 OK, EINVAL, EHIP, EUNSUPPORTED, ENOTFOUND, EIO = range(6)
+OPT_PAIRS, OPT_NO_BANK_RULE = 1, 2  # tetris_options_set
 
 
 class TetrisError(RuntimeError):
@@ -96,6 +97,8 @@ _lib.tetris_g950_create_device.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int
 _lib.tetris_g950_destroy.argtypes = [C.c_void_p]
 _lib.tetris_g950_destroy.restype = None
 _lib.tetris_g950_host_arrays.argtypes = [C.c_void_p, C.POINTER(_G950Arrays)]
+_lib.tetris_options_set.argtypes = [C.c_uint]
+_lib.tetris_options_get.restype = C.c_uint
 _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
 _lib.tetris_tile_table_load.argtypes = [C.c_char_p, C.POINTER(C.c_int)]
 _lib.tetris_measure_peaks.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
@@ -273,6 +276,15 @@ class G950Filter:
             self._h = None
 
     __del__ = close
+
+
+def options_set(flags):
+    """Ablation switches (OPT_PAIRS, OPT_NO_BANK_RULE) for launch plans made from now on."""
+    _check(_lib.tetris_options_set(flags))
+
+
+def options_get():
+    return int(_lib.tetris_options_get())
 
 
 def tile_select(batch, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding):
