@@ -204,8 +204,26 @@ size_t tetris_noalloc_scratch_bytes(void); /* bytes of the array the entry point
  * it); returns the limit now in force.  For harnesses that want a larger layer refused rather than run. */
 size_t tetris_noalloc_scratch_limit(size_t bytes);
 
-/* Same call shape as the reference launcher: the raw device arrays of a live tetris_spf (looked up by
- * `d_values`).  tile_h/tile_w are accepted for source compatibility and ignored. */
+/* The reference launcher on the five device arrays of a SparseFilter (Tetris/spconv2d_kernel.cuh:14-21,
+ * Tetris/spconv2d_kernel.cu:91-156): the convolution is computed FROM THE ARRAYS PASSED -- offsets, positions, values
+ * and the output-channel permutation -- not from anything a handle remembers.  The arrays are hashed on the device at
+ * every call (one pass over them and a stream synchronisation); the first call, and any call after their content has
+ * changed (a caller that rewrites d_values in place), decodes them on the device into the kernel's own pack, whose
+ * slots follow d_oc_permutation.  Decoded packs are cached per set of addresses (16 sets, least recently used first
+ * out).  d_stage_len is accepted and not read, as in the reference's kernel.  tile_ic and vec_width are the
+ * SparseFilter's TILE_IC (a template argument of the reference launcher) and entries per lane and step: 4
+ * (apply_vectorize), 1, or 0 for the keep-as-is layout of apply_reorder = false (spconv2d_utils.h:38-61; then
+ * d_oc_permutation may be NULL) -- the format of the reference's CSR-like baseline variant.  tile: NULL = the library
+ * chooses.  Not capturable into a HIP graph (it synchronises); capture tetris_spconv2d_launch instead. */
+int tetris_spconv2d_launch_spf_arrays(const float* d_input, const int32_t* d_offsets, const int32_t* d_stage_len,
+                                      const int32_t* d_oc_permutation, const int32_t* d_position, const float* d_values,
+                                      float* d_output, int batch, int img_h, int img_w, int in_channel, int out_channel,
+                                      int kernel_size, int stride, int padding, int tile_ic, int vec_width,
+                                      const tetris_tile* tile, void* stream);
+
+/* Same, in the exact call shape of the reference launcher, which carries neither TILE_IC nor the vector width:
+ * those two are taken from the live tetris_spf whose device arrays these are (found through d_values;
+ * TETRIS_ENOTFOUND otherwise).  The content still comes from the arrays. */
 int tetris_spconv2d_launch_spf(const float* d_input, const int32_t* d_offsets, const int32_t* d_stage_len,
                                const int32_t* d_oc_permutation, const int32_t* d_position, const float* d_values,
                                float* d_output, int batch, int img_h, int img_w, int in_channel, int out_channel,
@@ -219,13 +237,20 @@ int tetris_spconv2d_launch_spf(const float* d_input, const int32_t* d_offsets, c
  * protocol (30 warm-up + 100 timed launches between two events, Tetris/tensor_utils.h:10-11), and
  * download.  *ms_out (may be NULL) receives the mean milliseconds per launch.  `layout` is accepted
  * for source compatibility ("NHWC" in the reference's mains) and does not change the host layout.
+ * tetris_spconv2d_host lets the library choose the tile and, with apply_reorder, packs in the balanced channel order.
+ * tetris_spconv2d_spf_host follows the reference's fixed configuration instead: a SparseFilter with TILE_IC = 128,
+ * always reordered (spf.cc:43-44; apply_reorder is ignored there as here) and built with `flags` (the reference's
+ * -DBANK_OPTIMIZE / -DREORDER_OUT_CHANNEL), whose DEVICE ARRAYS feed the convolution (as
+ * tetris_spconv2d_launch_spf_arrays does), run with one fixed tile -- lanes over a quarter of the output width (at
+ * most 16), one quad, eight channels per wave, four waves, eight staged channels -- in place of <3, 1, 128, 2, 4>
+ * (spf.cc:59-60); a shape that tile cannot run gets the library's choice.
  * ---------------------------------------------------------------------------------------------- */
 int tetris_spconv2d_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
                          int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
                          void* stream, const char* layout, int apply_reorder, float* ms_out);
 int tetris_spconv2d_spf_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
                              int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
-                             void* stream, const char* layout, int apply_reorder, float* ms_out);
+                             void* stream, const char* layout, int apply_reorder, unsigned flags, float* ms_out);
 
 /* Times `repeat` back-to-back launches after `warm` untimed ones (TimingTetrisSparseConv2d,
  * Tetris/spconv2d.cc:29-69); mean milliseconds per launch in *ms_out. */

@@ -14,7 +14,7 @@
 // (Tetris/tensor_utils.cc:61-64).
 //
 // Differences a caller can see: device tensors are NCHW (the reference keeps NHWC on the device; the
-// host entry points take and return NCHW in both); the TILE_IC/TILE_H/TILE_W template arguments of
+// host entry points take and return NCHW in both); the TILE_H/TILE_W template arguments of
 // SparseConv2d are accepted and ignored (tile shapes are chosen by the library); the preprocessor
 // switches BANK_OPTIMIZE and REORDER_OUT_CHANNEL select the same variants as in the reference.
 #ifndef TETRIS_SPCONV2D_HPP_
@@ -105,19 +105,30 @@ struct SparseFilter {
   tetris_spf* handle_ = nullptr;
 };
 
-// The device arrays must belong to a live SparseFilter (the library finds its handle through `values`).
-// `input` and `output` are NCHW device tensors.  Asynchronous on `stream`.
+// Computes from the device arrays passed (offsets, positions, values, permutation), as the reference launcher does.
+// With TILE_IC given (the reference's callers always give the SparseFilter's own, Tetris/spf.cc:59-60) any arrays in
+// the SparseFilter layout work; without it they must belong to a live SparseFilter, whose TILE_IC is then looked up
+// through `values`.  TILE_H / TILE_W are accepted and ignored: the library picks its tile.  `input` and `output`
+// are NCHW device tensors.  The call hashes the arrays on the device and synchronises `stream` (a caller may have
+// rewritten them in place); the kernels run asynchronously.
 template <typename ValueType, typename OffsetType, typename PositionType, int KERNEL_SIZE = 0, int STRIDE = 0,
           int TILE_IC = 0, int TILE_H = 0, int TILE_W = 0, typename Stream = void*>
 void SparseConv2d(ValueType* input, OffsetType* offsets, OffsetType* stage_len, PositionType* oc_permutation,
                   PositionType* position, ValueType* values, ValueType* output, int batch_size, int img_h, int img_w,
                   int in_channel, int out_channel, int kernel_size, int stride, int padding, Stream stream) {
-  TETRIS_CHECK(tetris_spconv2d_launch_spf(input, reinterpret_cast<const int32_t*>(offsets),
-                                          reinterpret_cast<const int32_t*>(stage_len),
-                                          reinterpret_cast<const int32_t*>(oc_permutation),
-                                          reinterpret_cast<const int32_t*>(position), values, output, batch_size, img_h,
-                                          img_w, in_channel, out_channel, kernel_size, stride, padding,
-                                          reinterpret_cast<void*>(stream)));
+  if (TILE_IC > 0)
+    TETRIS_CHECK(tetris_spconv2d_launch_spf_arrays(
+        input, reinterpret_cast<const int32_t*>(offsets), reinterpret_cast<const int32_t*>(stage_len),
+        reinterpret_cast<const int32_t*>(oc_permutation), reinterpret_cast<const int32_t*>(position), values, output,
+        batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding, TILE_IC, 4, nullptr,
+        reinterpret_cast<void*>(stream)));
+  else
+    TETRIS_CHECK(tetris_spconv2d_launch_spf(input, reinterpret_cast<const int32_t*>(offsets),
+                                            reinterpret_cast<const int32_t*>(stage_len),
+                                            reinterpret_cast<const int32_t*>(oc_permutation),
+                                            reinterpret_cast<const int32_t*>(position), values, output, batch_size,
+                                            img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
+                                            reinterpret_cast<void*>(stream)));
 }
 
 // Prints the two result lines of the reference (Tetris/spconv2d.cc:357-358): milliseconds per launch and the
@@ -148,7 +159,7 @@ void SparseConv2d_SPF(float* h_input, float* h_filter, float* h_output, int batc
   float ms = 0.f;
   TETRIS_CHECK(tetris_spconv2d_spf_host(h_input, h_filter, h_output, batch_size, img_h, img_w, in_channel,
                                         out_channel, kernel_size, stride, padding, reinterpret_cast<void*>(stream),
-                                        layout.c_str(), apply_reorder, &ms));
+                                        layout.c_str(), apply_reorder, tetris_detail::build_flags(), &ms));
   std::cout << "Time of Ablation :" << ms << "ms"
             << "\n";
 }

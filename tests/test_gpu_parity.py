@@ -234,6 +234,93 @@ def test_reference_shaped_entry_points(env):
     assert e.value.code == T.ENOTFOUND
 
 
+def test_raw_launcher_computes_from_the_arrays_it_is_given(env):
+    # SparseConv2d<...> of the reference convolves whatever its five device arrays hold
+    # (Tetris/spconv2d_kernel.cuh:14-21, spconv2d_kernel.cu:91-156).  Arrays made by the ORACLE's packer (no library
+    # handle owns them) in every layout the constructor can produce -- plain / Bank-SR / Filter-GR / both, vector width
+    # 4 and 1, and the keep-as-is rows of apply_reorder = false -- must give the dense convolution; rewriting the values
+    # in place on the device must change the result of the next launch.
+    T, torch, O = env
+    N, C, H, W, K, ks, stride, pad = 2, 40, 17, 19, 70, 3, 1, 1
+    rng = np.random.default_rng(61)
+    w = sparse_filter(rng, K, C, ks, 0.8)
+    x = relu_like(rng, (N, C, H, W))
+    ref = O.host_conv2d(x, w, stride, pad, threads=4)
+    dx = torch.from_numpy(x).cuda()
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+
+    def launch(arrs, tile_ic, vec):
+        dy = torch.full((N, K, H, W), float("nan"), device="cuda")
+        T.SparseConv2d(dx.data_ptr(), arrs[0].data_ptr(), arrs[1].data_ptr() if arrs[1].numel() else 0, arrs[4].data_ptr(),
+                       arrs[2].data_ptr(), arrs[3].data_ptr(), dy.data_ptr(), N, H, W, C, K, ks, stride, pad, TILE_IC=tile_ic,
+                       vec_width=vec)
+        torch.cuda.synchronize()
+        return dy.cpu().numpy()
+
+    for tile_ic in (16, 128):
+        for bank, reoc, vec in [(0, 0, 4), (1, 0, 4), (0, 1, 4), (1, 1, 4), (1, 1, 1)]:
+            p = O.SpfPack(w, tile_ic, True, vec == 4, bool(bank), bool(reoc))
+            arrs = [dev(a) for a in p.arrays()]
+            assert max_rel_err(launch(arrs, tile_ic, vec), ref) <= TOL, (tile_ic, bank, reoc, vec)
+        p = O.SpfPack(w, tile_ic, False)  # keep-as-is rows: offsets per (channel, stage), no stage_len
+        arrs = [dev(a) for a in p.arrays()]
+        assert max_rel_err(launch(arrs, tile_ic, 0), ref) <= TOL
+    # in-place rewrite of the values on the device: same addresses, new content
+    p = O.SpfPack(w, 32, True, True, True, True)
+    arrs = [dev(a) for a in p.arrays()]
+    assert max_rel_err(launch(arrs, 32, 4), ref) <= TOL
+    arrs[3].mul_(-2.0)
+    torch.cuda.synchronize()
+    assert max_rel_err(launch(arrs, 32, 4), -2.0 * ref) <= TOL
+    # a permutation that is none is refused, and so are nonsense offsets
+    bad = [a.clone() for a in arrs]
+    bad[4].zero_()
+    with pytest.raises(T.TetrisError) as e:
+        launch(bad, 32, 4)
+    assert e.value.code == T.EINVAL
+
+
+def test_live_sparse_filter_arrays_rewritten_in_place(env):
+    # The reference-shaped call (no TILE_IC argument) on a live SparseFilter's device arrays: the handle only
+    # supplies TILE_IC; the weights are read from the device arrays at every launch.
+    T, torch, O = env
+    import ctypes
+    N, C, H, W, K, ks = 2, 24, 12, 12, 40, 3
+    rng = np.random.default_rng(62)
+    w = sparse_filter(rng, K, C, ks, 0.85)
+    x = relu_like(rng, (N, C, H, W))
+    ref = O.host_conv2d(x, w, 1, 1, threads=4)
+    sf = T.SparseFilter(w, C, K, ks, 64, True, True, T.BANK_OPTIMIZE | T.REORDER_OUT_CHANNEL)
+    dx = torch.from_numpy(x).cuda()
+    dy = torch.zeros((N, K, H, W), device="cuda")
+    args = (dx.data_ptr(), sf.GetDeviceOffsets(), sf.GetDeviceStageLen(), sf.GetDeviceOCPermutation(), sf.GetDevicePosition(),
+            sf.GetDeviceValues(), dy.data_ptr(), N, H, W, C, K, ks, 1, 1)
+    T.SparseConv2d(*args)
+    torch.cuda.synchronize()
+    assert max_rel_err(dy.cpu().numpy(), ref) <= TOL
+    hip = ctypes.CDLL("libamdhip64.so")
+    tripled = np.ascontiguousarray(3.0 * sf.values_)
+    assert hip.hipMemcpy(ctypes.c_void_p(sf.GetDeviceValues()), tripled.ctypes.data_as(ctypes.c_void_p),
+                         ctypes.c_size_t(tripled.nbytes), 1) == 0
+    T.SparseConv2d(*args)
+    torch.cuda.synchronize()
+    assert max_rel_err(dy.cpu().numpy(), 3.0 * ref) <= TOL
+    sf.close()
+
+
+@pytest.mark.parametrize("flags", [0, 1, 2, 3])
+def test_spf_entry_point_runs_the_fixed_configuration(env, flags):
+    # SparseConv2d_SPF: SparseFilter(TILE_IC = 128, always reordered) built with the given macros, its device arrays
+    # fed to the launcher, one fixed tile (Tetris/spf.cc:43-60)
+    T, torch, O = env
+    rng = np.random.default_rng(63 + flags)
+    for N, C, H, W, K, ks, stride, pad in [(2, 24, 20, 20, 48, 3, 1, 1), (1, 200, 9, 9, 36, 3, 1, 1), (3, 16, 14, 14, 32, 1, 1, 0)]:
+        w = sparse_filter(rng, K, C, ks, 0.85)
+        x = relu_like(rng, (N, C, H, W))
+        y, ms = T.SparseConv2d_SPF(x, w, N, H, W, C, K, ks, stride, pad, 0, "NHWC", False, flags)
+        assert ms > 0 and max_rel_err(y, O.host_conv2d(x, w, stride, pad, threads=4)) <= TOL
+
+
 @pytest.mark.parametrize("name", ["rn90_3x3", "rn90_stem", "rn98_1x1", "vgg_64x128", "yolo_255"])
 def test_shipped_pruned_layers(env, name):
     # real magnitude-pruned weights: very uneven rows, channels with no weights at all, K = 255

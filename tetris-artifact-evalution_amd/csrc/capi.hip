@@ -191,40 +191,201 @@ int time_launches(tetris_g950* p, const float* d_in, float* d_out, int N, int H,
   return done(TETRIS_OK);
 }
 
+// ---- the reference layout's device arrays as the source of a convolution ------------------------------------------
+// A view remembers, for one set of array addresses, the content hash it was built from, the dense filter decoded from
+// the arrays (device memory), and the kernel packs and tiles made from it.  At most kMaxViews live at a time.
+struct SpfView {
+  const void* ptrs[4];  // offsets, permutation, position, values
+  int C, K, ks, tile_ic, vec;
+  unsigned long long hash = 0;
+  float* d_filter = nullptr;
+  std::vector<int32_t> order;                              // oc_permutation copied to the host: the packs' slot order
+  std::map<std::array<int, 2>, tetris_g950*> packs;        // by (tile_ic of the kernel, oc_per_wave)
+  std::map<std::array<int, 5>, tetris_tile> tiles;         // by (N, H, W, stride, pad): the library's choice, made once
+  void clear() {
+    for (auto& kv : packs) tetris_g950_destroy(kv.second);
+    packs.clear();
+    tiles.clear();
+    if (d_filter) (void)hipFree(d_filter);
+    d_filter = nullptr;
+  }
+};
+constexpr size_t kMaxViews = 16;
+std::mutex g_views_mu;
+std::vector<SpfView*> g_views;  // most recently used last
+unsigned long long* g_hash_scratch = nullptr;
+
+void drop_views(const void* d_values) {
+  std::lock_guard<std::mutex> lock(g_views_mu);
+  for (size_t i = g_views.size(); i-- > 0;)
+    if (g_views[i]->ptrs[3] == d_values) {
+      g_views[i]->clear();
+      delete g_views[i];
+      g_views.erase(g_views.begin() + (long)i);
+    }
+}
+
+// The kernel pack (and tile) for a convolution whose weights are the arrays at these addresses, rebuilt when the
+// arrays' content has changed since the view was made.  Hashing reads the arrays once and synchronises `stream`.
+int view_pack(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_position, const float* d_values, int N,
+              int H, int W, int C, int K, int ks, int stride, int pad, int tile_ic, int vec, const tetris_tile* tile,
+              hipStream_t stream, tetris_g950** pack_out, tetris_tile* tile_out) {
+  if (!d_offsets || !d_position || !d_values || (vec != 0 && !d_perm)) return fail(TETRIS_EINVAL, "null argument");
+  if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || tile_ic <= 0 || (vec != 0 && vec != 1 && vec != 4))
+    return fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d tile_ic=%d vector width=%d", C, K, ks, tile_ic, vec);
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+    return fail(TETRIS_EINVAL, "this entry point reads the arrays back (a synchronisation): it cannot be captured; "
+                "capture tetris_spconv2d_launch on a tetris_g950 instead");
+  const int stages = (C - 1) / tile_ic + 1;
+  const int n_off = (vec == 0 ? K : (K + kRefLanes - 1) / kRefLanes) * stages + 1;
+  std::lock_guard<std::mutex> lock(g_views_mu);
+  if (!g_hash_scratch) TETRIS_HIP(hipMalloc(&g_hash_scratch, 16));
+  unsigned long long hash = 0;
+  long long n_ent = 0;
+  int rc = spf_arrays_hash(d_offsets, n_off, d_perm, vec == 0 ? 0 : K, d_position, d_values, vec == 0 ? 1 : kRefLanes,
+                           g_hash_scratch, stream, &hash, &n_ent);
+  if (rc) return rc;
+  if (n_ent < 0 || n_ent > (1ll << 31)) return fail(TETRIS_EINVAL, "offsets end at %lld entries: not a packed filter", n_ent);
+  hash ^= 0x5bd1e995ull * (unsigned long long)(C * 131 + ks) + (unsigned long long)tile_ic * 7919ull + (unsigned)vec;
+  SpfView* v = nullptr;
+  for (size_t i = 0; i < g_views.size(); ++i) {
+    SpfView* c = g_views[i];
+    if (c->ptrs[0] == d_offsets && c->ptrs[1] == d_perm && c->ptrs[2] == d_position && c->ptrs[3] == d_values && c->C == C &&
+        c->K == K && c->ks == ks && c->tile_ic == tile_ic && c->vec == vec) {
+      v = c;
+      g_views.erase(g_views.begin() + (long)i);
+      break;
+    }
+  }
+  if (!v) {
+    v = new SpfView;
+    v->ptrs[0] = d_offsets; v->ptrs[1] = d_perm; v->ptrs[2] = d_position; v->ptrs[3] = d_values;
+    v->C = C; v->K = K; v->ks = ks; v->tile_ic = tile_ic; v->vec = vec;
+    v->hash = ~hash;
+  }
+  g_views.push_back(v);
+  while (g_views.size() > kMaxViews) {
+    g_views.front()->clear();
+    delete g_views.front();
+    g_views.erase(g_views.begin());
+  }
+  if (v->hash != hash || !v->d_filter) {  // new, or rewritten in place since the view was made: decode again
+    v->clear();
+    TETRIS_HIP(hipMalloc(&v->d_filter, sizeof(float) * (size_t)C * K * ks * ks));
+    rc = spf_arrays_decode(d_offsets, d_perm, d_position, d_values, v->d_filter, C, K, ks, tile_ic, vec, stream);
+    if (rc) return rc;
+    v->order.assign(K, 0);
+    if (vec != 0) {
+      TETRIS_HIP(hipMemcpyAsync(v->order.data(), d_perm, sizeof(int32_t) * K, hipMemcpyDeviceToHost, stream));
+      TETRIS_HIP(hipStreamSynchronize(stream));
+      std::vector<char> seen(K, 0);
+      for (int k = 0; k < K; ++k) {
+        if (v->order[k] < 0 || v->order[k] >= K || seen[v->order[k]])
+          return fail(TETRIS_EINVAL, "oc_permutation is not a permutation of 0..%d", K - 1);
+        seen[v->order[k]] = 1;
+      }
+    } else {
+      for (int k = 0; k < K; ++k) v->order[k] = k;
+    }
+    v->hash = hash;
+  }
+  tetris_tile t{};
+  if (tile && tile->lanes_w > 0) {
+    t = *tile;
+  } else {
+    const std::array<int, 5> key{N, H, W, stride, pad};
+    auto it = v->tiles.find(key);
+    if (it == v->tiles.end()) {
+      rc = choose_tile(N, H, W, C, K, ks, stride, pad, &t);
+      if (rc) return rc;
+      it = v->tiles.emplace(key, t).first;
+    }
+    t = it->second;
+  }
+  const std::array<int, 2> pkey{t.tile_ic, t.oc_per_wave};
+  auto it = v->packs.find(pkey);
+  if (it == v->packs.end()) {
+    // slots in the order of the arrays' own oc_permutation: the caller's channel regrouping is kept
+    tetris_g950* p = nullptr;
+    rc = tetris_g950_create_device(v->d_filter, C, K, ks, t.tile_ic, t.oc_per_wave, v->order.data(), stream, &p);
+    if (rc) return rc;
+    it = v->packs.emplace(pkey, p).first;
+  }
+  *pack_out = it->second;
+  *tile_out = t;
+  return TETRIS_OK;
+}
+
 // Shared body of the two host-to-host entry points.
+// The fixed tile of the spf entry point, the counterpart of the reference's one instantiation <3, 1, 128, 2, 4>
+// (Tetris/spf.cc:59-60): four waves of eight channels, one quad, eight staged channels, lanes across a quarter of the
+// output width (at most 16).  A shape it cannot run falls back to the library's choice.
+tetris_tile fixed_spf_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad) {
+  tetris_tile t{};
+  const int OW = out_extent(W, pad, ks, stride);
+  t.lanes_w = std::max(1, std::min(16, ceil_div(OW, 4)));
+  t.quads = 1; t.oc_per_wave = 8; t.waves = 4; t.tile_ic = std::min(8, C);
+  tetris_g950 shape;
+  shape.C = C; shape.K = K; shape.ks = ks; shape.tile_ic = t.tile_ic; shape.g = t.oc_per_wave;
+  shape.stages = ceil_div(C, t.tile_ic);
+  shape.slots = ceil_div(K, kSlotPad) * kSlotPad;
+  Geom g;
+  if (make_geom(&shape, N, H, W, stride, pad, t, &g) != TETRIS_OK) (void)choose_tile(N, H, W, C, K, ks, stride, pad, &t);
+  return t;
+}
+
+// Shared body of the two host-to-host entry points.  spf_path: the reference's SparseConv2d_SPF (Tetris/spf.cc:22-93):
+// SparseFilter with TILE_IC = 128 and apply_reorder = true whatever the caller passed (:43-44), its device arrays handed
+// to the launcher, one fixed tile.
 int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K, int ks,
-              int stride, int pad, hipStream_t stream, bool apply_reorder, bool fixed_spf_config, float* ms_out) {
+              int stride, int pad, hipStream_t stream, bool apply_reorder, bool spf_path, unsigned spf_flags,
+              float* ms_out) {
   if (!h_in || !h_filter || !h_out) return fail(TETRIS_EINVAL, "null argument");
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad conv shape");
   const int OH = out_extent(H, pad, ks, stride), OW = out_extent(W, pad, ks, stride);
   if (OH <= 0 || OW <= 0) return fail(TETRIS_EINVAL, "empty output");
   tetris_tile tile{};
-  int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &tile);
-  if (rc) return rc;
-  // apply_reorder: the reference regroups output channels for its warps (ReorderOutChannel); the kernel here
-  // gets the order that balances its own waves instead.  The results do not depend on the order.
-  // The reference's spf entry point fixes its tile template arguments; here both entry points leave the
-  // tile to the selector.
-  (void)fixed_spf_config;
-  std::vector<int32_t> order;
-  if (apply_reorder) {
-    order.resize(K);
-    rc = balance_oc_order(h_filter, C, K, ks, tile, order.data());
-    if (rc) return rc;
-  }
-  tetris_g950* pack = nullptr;
-  rc = tetris_g950_create(h_filter, C, K, ks, tile.tile_ic, tile.oc_per_wave, apply_reorder ? order.data() : nullptr,
-                          stream, &pack);
+  tetris_g950* pack = nullptr;   // owned here (the normal path)
+  tetris_spf* spf = nullptr;     // owned here (the spf path; its view owns the pack)
   float *d_in = nullptr, *d_out = nullptr;
   const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
   auto done = [&](int code) {
     if (d_in) (void)hipFree(d_in);
     if (d_out) (void)hipFree(d_out);
     tetris_g950_destroy(pack);
+    tetris_spf_destroy(spf);
     return code;
   };
-  if (rc) return done(rc);
+  int rc;
+  tetris_g950* run = nullptr;
+  if (spf_path) {
+    rc = tetris_spf_create(h_filter, C, K, ks, 128, 1, 1, spf_flags, &spf);
+    if (rc) return done(rc);
+    tetris_spf_arrays a{};
+    rc = tetris_spf_device_arrays(spf, &a);
+    if (rc) return done(rc);
+    const tetris_tile fixed = fixed_spf_tile(N, H, W, C, K, ks, stride, pad);
+    rc = view_pack(a.offsets, a.oc_permutation, a.position, a.values, N, H, W, C, K, ks, stride, pad, 128, 4, &fixed, stream,
+                   &run, &tile);
+    if (rc) return done(rc);
+  } else {
+    rc = choose_tile(N, H, W, C, K, ks, stride, pad, &tile);
+    if (rc) return done(rc);
+    // apply_reorder: the reference regroups output channels for its warps (ReorderOutChannel); the kernel here
+    // gets the order that balances its own waves instead.  The results do not depend on the order.
+    std::vector<int32_t> order;
+    if (apply_reorder) {
+      order.resize(K);
+      rc = balance_oc_order(h_filter, C, K, ks, tile, order.data());
+      if (rc) return done(rc);
+    }
+    rc = tetris_g950_create(h_filter, C, K, ks, tile.tile_ic, tile.oc_per_wave, apply_reorder ? order.data() : nullptr,
+                            stream, &pack);
+    if (rc) return done(rc);
+    run = pack;
+  }
 #define HIPD(call)                                                                                          \
   do {                                                                                                      \
     hipError_t e_ = (call);                                                                                 \
@@ -235,7 +396,7 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
   HIPD(hipMalloc(&d_out, out_bytes));
   HIPD(hipMemcpyAsync(d_in, h_in, in_bytes, hipMemcpyHostToDevice, stream));
   float ms = 0;
-  rc = time_launches(pack, d_in, d_out, N, H, W, stride, pad, &tile, stream, 30, 100, &ms);
+  rc = time_launches(run, d_in, d_out, N, H, W, stride, pad, &tile, stream, 30, 100, &ms);
   if (rc) return done(rc);
   HIPD(hipMemcpyAsync(h_out, d_out, out_bytes, hipMemcpyDeviceToHost, stream));
   HIPD(hipStreamSynchronize(stream));
@@ -278,24 +439,6 @@ static int spf_ensure_device(tetris_spf* f) {
   return TETRIS_OK;
 }
 
-// The kernel's own pack of this filter for tile `t`, with the output-channel order that balances the tile's waves.
-static int spf_kernel_pack(tetris_spf* f, const tetris_tile& t, hipStream_t stream, tetris_g950** out) {
-  std::lock_guard<std::mutex> lock(f->mu);
-  const std::array<int, 3> key{t.tile_ic, t.oc_per_wave, t.waves};
-  auto it = f->kernel_packs.find(key);
-  if (it == f->kernel_packs.end()) {
-    std::vector<int32_t> order(f->K);
-    int rc = balance_oc_order(f->filter.data(), f->C, f->K, f->ks, t, order.data());
-    if (rc) return rc;
-    tetris_g950* p = nullptr;
-    rc = tetris_g950_create(f->filter.data(), f->C, f->K, f->ks, t.tile_ic, t.oc_per_wave, order.data(), stream, &p);
-    if (rc) return rc;
-    it = f->kernel_packs.emplace(key, p).first;
-  }
-  *out = it->second;
-  return TETRIS_OK;
-}
-
 int tetris_spf_create(const float* h_filter, int C, int K, int ks, int tile_ic, int apply_reorder, int apply_vectorize,
                       unsigned flags, tetris_spf** out) {
   if (!out) return fail(TETRIS_EINVAL, "null argument");
@@ -305,7 +448,7 @@ int tetris_spf_create(const float* h_filter, int C, int K, int ks, int tile_ic, 
     delete f;
     return rc;
   }
-  f->filter.assign(h_filter, h_filter + (size_t)C * K * ks * ks);  // the kernel's packs are made from it at launch
+  f->vec = apply_reorder ? (apply_vectorize ? 4 : 1) : 0;
   *out = f;
   return TETRIS_OK;
 }
@@ -317,7 +460,7 @@ void tetris_spf_destroy(tetris_spf* f) {
     auto it = g_registry.find(f->d_values);
     if (it != g_registry.end() && it->second == f) g_registry.erase(it);
   }
-  for (auto& kv : f->kernel_packs) tetris_g950_destroy(kv.second);
+  drop_views(f->d_values);
   if (f->d_offsets) (void)hipFree(f->d_offsets);
   if (f->d_stage_len) (void)hipFree(f->d_stage_len);
   if (f->d_position) (void)hipFree(f->d_position);
@@ -500,27 +643,41 @@ int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_in, float* d_o
   return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, stream);
 }
 
+int tetris_spconv2d_launch_spf_arrays(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,
+                                      const int32_t* d_perm, const int32_t* d_position, const float* d_values,
+                                      float* d_out, int N, int H, int W, int C, int K, int ks, int stride, int pad,
+                                      int tile_ic, int vec_width, const tetris_tile* tile, void* stream_) {
+  (void)d_stage_len;  // the reference's kernel does not read it either (Tetris/spconv2d_kernel.cu:13-160)
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  tetris_g950* pack = nullptr;
+  tetris_tile t{};
+  int rc = view_pack(d_offsets, d_perm, d_position, d_values, N, H, W, C, K, ks, stride, pad, tile_ic, vec_width, tile, stream,
+                     &pack, &t);
+  if (rc) return rc;
+  return run_launch(pack, d_in, d_out, N, H, W, stride, pad, &t, stream);
+}
+
 int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,
                                const int32_t* d_perm, const int32_t* d_position, const float* d_values, float* d_out,
                                int N, int H, int W, int C, int K, int ks, int stride, int pad, void* stream) {
-  (void)d_offsets; (void)d_stage_len; (void)d_perm; (void)d_position;
-  tetris_spf* f = nullptr;
+  // the call shape of the reference launcher carries neither TILE_IC (a template argument there) nor the vector
+  // width: they are taken from the live tetris_spf that owns `d_values`; the CONTENT comes from the arrays
+  int tile_ic = 0, vec = 0;
   {
     std::lock_guard<std::mutex> lock(g_registry_mu);
     auto it = g_registry.find(d_values);
-    if (it != g_registry.end()) f = it->second;
+    if (it == g_registry.end())
+      return fail(TETRIS_ENOTFOUND, "device arrays do not belong to a live tetris_spf handle (use "
+                  "tetris_spconv2d_launch_spf_arrays for arrays of your own)");
+    const tetris_spf* f = it->second;
+    if (f->C != C || f->K != K || f->ks != ks)
+      return fail(TETRIS_EINVAL, "shape C=%d K=%d ks=%d does not match the packed filter (%d, %d, %d)", C, K, ks, f->C,
+                  f->K, f->ks);
+    tile_ic = f->tile_ic;
+    vec = f->vec;
   }
-  if (!f) return fail(TETRIS_ENOTFOUND, "device arrays do not belong to a live tetris_spf handle");
-  if (f->C != C || f->K != K || f->ks != ks)
-    return fail(TETRIS_EINVAL, "shape C=%d K=%d ks=%d does not match the packed filter (%d, %d, %d)", C, K, ks, f->C,
-                f->K, f->ks);
-  tetris_tile t{};
-  int rc = choose_tile(N, H, W, C, K, ks, stride, pad, &t);
-  if (rc) return rc;
-  tetris_g950* pack = nullptr;
-  rc = spf_kernel_pack(f, t, static_cast<hipStream_t>(stream), &pack);
-  if (rc) return rc;
-  return run_launch(pack, d_in, d_out, N, H, W, stride, pad, &t, static_cast<hipStream_t>(stream));
+  return tetris_spconv2d_launch_spf_arrays(d_in, d_offsets, d_stage_len, d_perm, d_position, d_values, d_out, N, H, W, C,
+                                           K, ks, stride, pad, tile_ic, vec, nullptr, stream);
 }
 
 int tetris_spconv2d_time(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
@@ -534,15 +691,17 @@ int tetris_spconv2d_host(const float* h_in, const float* h_filter, float* h_out,
                          float* ms_out) {
   (void)layout;
   return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream),
-                   apply_reorder != 0, false, ms_out);
+                   apply_reorder != 0, false, 0u, ms_out);
 }
 
 int tetris_spconv2d_spf_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K,
                              int ks, int stride, int pad, void* stream, const char* layout, int apply_reorder,
-                             float* ms_out) {
+                             unsigned flags, float* ms_out) {
   (void)layout;
-  return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream),
-                   apply_reorder != 0, true, ms_out);
+  (void)apply_reorder;  // the reference ignores it here too: its SparseFilter is always built reordered (spf.cc:43-44)
+  if (flags & ~(TETRIS_BANK_OPTIMIZE | TETRIS_REORDER_OUT_CHANNEL)) return fail(TETRIS_EINVAL, "unknown flags 0x%x", flags);
+  return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream), true, true,
+                   flags, ms_out);
 }
 
 int tetris_read_weight_file(const char* path, int32_t header[8], float** h_filter_out, int64_t* nnz_out) {

@@ -197,8 +197,7 @@ struct tetris_spf {
   std::vector<float> values;
   int32_t *d_offsets = nullptr, *d_stage_len = nullptr, *d_position = nullptr, *d_oc_permutation = nullptr;
   float* d_values = nullptr;
-  std::vector<float> filter;                              // dense copy the kernel's packs are made from
-  std::map<std::array<int, 3>, tetris_g950*> kernel_packs;  // by (staged input channels, slots per wave, waves)
+  int vec = 0;  // entries per lane and step in `position` / `values`: 4, 1, or 0 for the keep-as-is layout
   std::mutex mu;
 };
 
@@ -212,6 +211,13 @@ int spf_pack_host(const float* filter, int C, int K, int ks, int tile_ic, bool a
 // entries of the pack bound to geometry `g`; paired: rearranged into pairs and singles (kernels that walk pairs)
 int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, const int2** entries_out,
               const int32_t** grp_off_out, const int32_t** grp_pair_out);
+
+// spf_pack_device.hip: the reference layout's device arrays as the source of a convolution
+int spf_arrays_hash(const int32_t* d_offsets, int n_off, const int32_t* d_perm, int K, const int32_t* d_position,
+                    const float* d_values, int lanes, unsigned long long* d_scratch2, hipStream_t stream,
+                    unsigned long long* hash_out, long long* n_ent_out);
+int spf_arrays_decode(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_position, const float* d_values,
+                      float* d_filter, int C, int K, int ks, int tile_ic, int vec, hipStream_t stream);
 
 // tile_select.cpp
 unsigned options();  // TETRIS_OPT_* flags in force (tetris_options_set, or the environment variable TETRIS_OPTIONS)

@@ -353,6 +353,109 @@ int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, co
   return TETRIS_OK;
 }
 
+// ---- the reference layout's device arrays as the source of a convolution ------------------------------------------
+// SparseConv2d<...> of the reference computes from offsets_/position_/values_/oc_permutation_ on the device
+// (Tetris/spconv2d_kernel.cu:91-156).  Here those arrays are decoded, on the device, back into a dense OIHW filter
+// from which the kernel's own pack is made; a content hash tells when a caller has rewritten them in place.
+namespace {
+
+__device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+// out[0] += order-independent hash of (array id, index, word) over the four arrays; out[1] = entry count
+__global__ __launch_bounds__(256) void spf_hash_kernel(const int32_t* __restrict__ offsets, int n_off,
+                                                       const int32_t* __restrict__ perm, int K,
+                                                       const int32_t* __restrict__ position,
+                                                       const float* __restrict__ values, int lanes,
+                                                       unsigned long long* __restrict__ out) {
+  const long long n_ent = (long long)lanes * offsets[n_off - 1];
+  const long long total = n_off + K + 2 * n_ent;
+  unsigned long long h = 0;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+    unsigned word;
+    if (i < n_off) word = (unsigned)offsets[i];
+    else if (i < n_off + K) word = (unsigned)perm[i - n_off];
+    else if (i < n_off + K + n_ent) word = (unsigned)position[i - n_off - K];
+    else word = __float_as_uint(values[i - n_off - K - n_ent]);
+    h += mix64(((unsigned long long)i << 32) ^ word ^ 0x9E3779B97F4A7C15ull);
+  }
+  for (int off = 32; off > 0; off >>= 1) h += __shfl_xor(h, off);
+  if ((threadIdx.x & 63) == 0) atomicAdd(out, h);
+  if (blockIdx.x == 0 && threadIdx.x == 0) out[1] = (unsigned long long)n_ent;
+}
+
+// vec > 0: the reorder path's layout (Tetris/spconv2d_utils.h:206-244): one workgroup per (32-lane group, stage);
+// entry e of lane l sits at 32 * offsets[seg] + (e / vec) * 32 * vec + l * vec + e % vec and belongs to output channel
+// perm[group * 32 + l], input channel (position >> 6) + stage * tile_ic.  vec == 0: the keep-as-is layout (:38-61),
+// one run of entries per (output channel, stage).  Zero values (padding of either kind) are skipped.
+__global__ __launch_bounds__(256) void spf_decode_kernel(const int32_t* __restrict__ offsets,
+                                                         const int32_t* __restrict__ perm,
+                                                         const int32_t* __restrict__ position,
+                                                         const float* __restrict__ values, float* __restrict__ filter,
+                                                         int C, int K, int ks, int tile_ic, int stages, int vec) {
+  const int seg = blockIdx.x;
+  const int stage = seg % stages, row = seg / stages;  // row: 32-lane group, or output channel when vec == 0
+  const int beg = offsets[seg], len = offsets[seg + 1] - beg;
+  const int kk = ks * ks;
+  if (vec == 0) {
+    for (int e = threadIdx.x; e < len; e += blockDim.x) {
+      const float v = values[beg + e];
+      const int pos = position[beg + e];
+      const int c = (pos >> 6) + stage * tile_ic, r = (pos >> 3) & 7, s_ = pos & 7;
+      if (v != 0.f && c < C && r < ks && s_ < ks) filter[((size_t)row * C + c) * kk + r * ks + s_] = v;
+    }
+    return;
+  }
+  const long long base = 32ll * beg;
+  for (int j = threadIdx.x; j < 32 * len; j += blockDim.x) {
+    const int lane = (j % (32 * vec)) / vec;
+    const int slot = row * 32 + lane;
+    const float v = values[base + j];
+    if (slot >= K || v == 0.f) continue;
+    const int pos = position[base + j];
+    const int c = (pos >> 6) + stage * tile_ic, r = (pos >> 3) & 7, s_ = pos & 7;
+    const int k = perm[slot];
+    if (k >= 0 && k < K && c < C && r < ks && s_ < ks) filter[((size_t)k * C + c) * kk + r * ks + s_] = v;
+  }
+}
+
+__global__ void fill_zero_kernel(float* __restrict__ p, long long n) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) p[i] = 0.f;
+}
+
+}  // namespace
+
+int spf_arrays_hash(const int32_t* d_offsets, int n_off, const int32_t* d_perm, int K, const int32_t* d_position,
+                    const float* d_values, int lanes, unsigned long long* d_scratch2, hipStream_t stream,
+                    unsigned long long* hash_out, long long* n_ent_out) {
+  hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<float*>(d_scratch2), 4ll);
+  hipLaunchKernelGGL(spf_hash_kernel, dim3(256), dim3(256), 0, stream, d_offsets, n_off, d_perm, K, d_position, d_values,
+                     lanes, d_scratch2);
+  TETRIS_HIP(hipGetLastError());
+  unsigned long long h[2] = {0, 0};
+  TETRIS_HIP(hipMemcpyAsync(h, d_scratch2, sizeof h, hipMemcpyDeviceToHost, stream));
+  TETRIS_HIP(hipStreamSynchronize(stream));
+  *hash_out = h[0];
+  *n_ent_out = (long long)h[1];
+  return TETRIS_OK;
+}
+
+int spf_arrays_decode(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_position, const float* d_values,
+                      float* d_filter, int C, int K, int ks, int tile_ic, int vec, hipStream_t stream) {
+  const int stages = (C - 1) / tile_ic + 1;
+  const int rows = vec == 0 ? K : (K + 31) / 32;
+  const long long n = (long long)C * K * ks * ks;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)std::min<long long>((n + 255) / 256, 4096)), dim3(256), 0, stream,
+                     d_filter, n);
+  hipLaunchKernelGGL(spf_decode_kernel, dim3(rows * stages), dim3(256), 0, stream, d_offsets, d_perm, d_position, d_values,
+                     d_filter, C, K, ks, tile_ic, stages, vec);
+  TETRIS_HIP(hipGetLastError());
+  return TETRIS_OK;
+}
+
 }  // namespace tetris
 
 extern "C" {

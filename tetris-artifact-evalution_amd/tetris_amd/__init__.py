@@ -115,9 +115,11 @@ _lib.tetris_noalloc_scratch_limit.restype = C.c_size_t
 _lib.tetris_spconv2d_launch_spf.argtypes = [C.c_void_p] * 7 + [C.c_int] * 8 + [C.c_void_p]
 _lib.tetris_spconv2d_time.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
     C.POINTER(Tile), C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float)]
-for _n in ("tetris_spconv2d_host", "tetris_spconv2d_spf_host"):
-    getattr(_lib, _n).argtypes = [_f32p, _f32p, _f32p] + [C.c_int] * 8 + [C.c_void_p, C.c_char_p, C.c_int,
-                                                                          C.POINTER(C.c_float)]
+_lib.tetris_spconv2d_launch_spf_arrays.argtypes = [C.c_void_p] * 7 + [C.c_int] * 10 + [C.POINTER(Tile), C.c_void_p]
+_lib.tetris_spconv2d_host.argtypes = [_f32p, _f32p, _f32p] + [C.c_int] * 8 + [C.c_void_p, C.c_char_p, C.c_int,
+                                                                            C.POINTER(C.c_float)]
+_lib.tetris_spconv2d_spf_host.argtypes = [_f32p, _f32p, _f32p] + [C.c_int] * 8 + [C.c_void_p, C.c_char_p, C.c_int, C.c_uint,
+                                                                                C.POINTER(C.c_float)]
 _lib.tetris_read_weight_file.argtypes = [C.c_char_p, C.POINTER(C.c_int32), C.POINTER(C.POINTER(C.c_float)),
                                          C.POINTER(C.c_int64)]
 _lib.tetris_free.argtypes = [C.c_void_p]
@@ -339,23 +341,31 @@ def tile_autotune(filter, batch, img_h, img_w, stride, padding, max_candidates=0
 
 
 def SparseConv2d(input, offsets, stage_len, oc_permutation, position, values, output, batch_size, img_h, img_w,
-                 in_channel, out_channel, kernel_size, stride, padding, stream=0):
-    """The reference launcher's call shape on raw device pointers of a live SparseFilter."""
-    _check(_lib.tetris_spconv2d_launch_spf(C.c_void_p(input), C.c_void_p(offsets), C.c_void_p(stage_len),
-                                           C.c_void_p(oc_permutation), C.c_void_p(position), C.c_void_p(values),
-                                           C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel,
-                                           kernel_size, stride, padding, C.c_void_p(stream)))
+                 in_channel, out_channel, kernel_size, stride, padding, stream=0, TILE_IC=0, vec_width=4, tile=None):
+    """The reference launcher's call shape on raw device pointers: computes from the arrays passed.  TILE_IC = 0: the
+    arrays belong to a live SparseFilter, whose TILE_IC is looked up; else any arrays in that layout
+    (vec_width 4, 1, or 0 for the keep-as-is layout of apply_reorder=False)."""
+    if TILE_IC:
+        _check(_lib.tetris_spconv2d_launch_spf_arrays(
+            C.c_void_p(input), C.c_void_p(offsets), C.c_void_p(stage_len), C.c_void_p(oc_permutation), C.c_void_p(position),
+            C.c_void_p(values), C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
+            padding, TILE_IC, vec_width, C.byref(tile) if tile is not None else None, C.c_void_p(stream)))
+    else:
+        _check(_lib.tetris_spconv2d_launch_spf(C.c_void_p(input), C.c_void_p(offsets), C.c_void_p(stage_len),
+                                               C.c_void_p(oc_permutation), C.c_void_p(position), C.c_void_p(values),
+                                               C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel,
+                                               kernel_size, stride, padding, C.c_void_p(stream)))
 
 
 def _host_entry(fn, h_input, h_filter, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
-                stream, layout, apply_reorder):
+                stream, layout, apply_reorder, *extra):
     x = np.ascontiguousarray(h_input, np.float32)
     w = np.ascontiguousarray(h_filter, np.float32)
     out = np.empty((batch_size, out_channel, out_extent(img_h, padding, kernel_size, stride),
                     out_extent(img_w, padding, kernel_size, stride)), np.float32)
     ms = C.c_float()
     _check(fn(x, w, out, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
-              C.c_void_p(stream), layout.encode(), int(apply_reorder), C.byref(ms)))
+              C.c_void_p(stream), layout.encode(), int(apply_reorder), *extra, C.byref(ms)))
     return out, float(ms.value)
 
 
@@ -367,9 +377,11 @@ def CudaSparseConv2d(h_input, h_filter, batch_size, img_h, img_w, in_channel, ou
 
 
 def SparseConv2d_SPF(h_input, h_filter, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
-                     padding, stream=0, layout="NHWC", apply_reorder=True):
+                     padding, stream=0, layout="NHWC", apply_reorder=True, flags=BANK_OPTIMIZE | REORDER_OUT_CHANNEL):
+    """The reference's fixed configuration (spf.cc): SparseFilter(TILE_IC=128, reordered, `flags`), its device arrays
+    fed to the launcher, one fixed tile."""
     return _host_entry(_lib.tetris_spconv2d_spf_host, h_input, h_filter, batch_size, img_h, img_w, in_channel,
-                       out_channel, kernel_size, stride, padding, stream, layout, apply_reorder)
+                       out_channel, kernel_size, stride, padding, stream, layout, apply_reorder, flags)
 
 
 def ReadConfigAndDataFromFile(weight_file):
