@@ -579,6 +579,55 @@ def test_prepare_then_capture_without_an_eager_launch(env):
     other.close()
 
 
+def test_autotune_and_timing_entry_points(env):
+    # tetris_tile_autotune (GetTetrisSparseConv2dTime, Tetris/spconv2d.cc:72-329) and tetris_spconv2d_time
+    # (TimingTetrisSparseConv2d, :29-69): the measured tile launches, computes the right thing and is not slower than
+    # the unmeasured choice; the exhaustive mode (every legal tile, the reference's table walk :285-329) is at least as
+    # good as a short candidate list; the timing loop agrees with events recorded around the same launches.
+    T, torch, O = env
+    rng = np.random.default_rng(71)
+    N, C, H, W, K, ks, stride, pad = 4, 48, 28, 28, 96, 3, 1, 1
+    w = sparse_filter(rng, K, C, ks, 0.85)
+    x = relu_like(rng, (N, C, H, W))
+    ref = O.host_conv2d(x, w, stride, pad, threads=8)
+    dx = torch.from_numpy(x).cuda()
+    dy = torch.empty((N, K, H, W), device="cuda")
+
+    def timed(tile):
+        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+        y = run_conv(T, torch, pk, x, K, ks, stride, pad, tile)
+        assert max_rel_err(y, ref) <= TOL, tile
+        ms = min(pk.time(dx.data_ptr(), dy.data_ptr(), N, H, W, stride, pad, tile, warm=10, repeat=50) for _ in range(3))
+        return pk, ms
+
+    tuned, ms_tuned = T.tile_autotune(w, N, H, W, stride, pad, 16)
+    assert ms_tuned > 0 and tuned.lanes_w >= 1
+    pk_t, t_tuned = timed(tuned)
+    pk_s, t_sel = timed(T.tile_select(N, H, W, C, K, ks, stride, pad))
+    assert t_tuned <= 1.15 * t_sel, (t_tuned, t_sel)
+    full, ms_full = T.tile_autotune(w, N, H, W, stride, pad, -1)  # exhaustive
+    pk_f, t_full = timed(full)
+    assert ms_full > 0 and t_full <= 1.15 * t_tuned, (t_full, t_tuned)
+    # the timing loop against events of our own around the same number of launches
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(10):
+        pk_t.launch(dx.data_ptr(), dy.data_ptr(), N, H, W, stride, pad, tuned)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(50):
+        pk_t.launch(dx.data_ptr(), dy.data_ptr(), N, H, W, stride, pad, tuned)
+    e1.record()
+    torch.cuda.synchronize()
+    assert 0.6 * t_tuned <= e0.elapsed_time(e1) / 50 <= 1.6 * t_tuned
+    with pytest.raises(T.TetrisError) as e:
+        pk_t.time(dx.data_ptr(), dy.data_ptr(), N, H, W, stride, pad, tuned, warm=1, repeat=0)
+    assert e.value.code == T.EINVAL
+    with pytest.raises(T.TetrisError):
+        T.tile_autotune(w, 0, H, W, stride, pad, 4)
+    for pk in (pk_t, pk_s, pk_f):
+        pk.close()
+
+
 def test_measured_ceilings_are_plausible(env):
     T, torch, O = env
     copy_gbs, fma_tflops = T.measure_peaks()

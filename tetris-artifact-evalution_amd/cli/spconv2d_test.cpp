@@ -127,6 +127,7 @@ int main(int argc, char* argv[]) {
 #endif
   CLI_HIP(hipStreamDestroy(stream));
 
+  int exit_code = 0;
   if (check) {  // what the reference's mains do when not built with -DBENCHMARK (Tetris/spconv2d.cc:430-440)
     float* h_check = static_cast<float*>(std::malloc(n_out * sizeof(float)));
     if (!h_check) {
@@ -137,8 +138,10 @@ int main(int argc, char* argv[]) {
     HostConv2d(h_input, h_filter, h_check, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
                padding);
     std::cout << "HostConv2d end\n";
-    std::cout << (TensorEqual(h_sparse, h_check, n_out) ? "Sparse Pass.\n" : "Sparse Error.\n");
+    const bool same = TensorEqual(h_sparse, h_check, n_out);
+    std::cout << (same ? "Sparse Pass.\n" : "Sparse Error.\n");
     std::free(h_check);
+    if (!same) exit_code = 3;  // the reference only prints the verdict; a script gets it from the exit status here
   }
 
   if (!dump.empty()) {
@@ -153,5 +156,5 @@ int main(int argc, char* argv[]) {
   std::free(h_input);
   std::free(h_filter);
   std::free(h_sparse);
-  return 0;
+  return exit_code;
 }

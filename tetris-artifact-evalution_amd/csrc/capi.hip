@@ -522,8 +522,12 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
                          int max_candidates, void* stream_, tetris_tile* out, float* ms_out) {
   if (!h_filter || !out) return fail(TETRIS_EINVAL, "null argument");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs) return fail(TETRIS_EINVAL, "bad layer shape");
+  size_t nnz = 0;
+  const size_t n_w = (size_t)C * K * ks * ks;
+  for (size_t i = 0; i < n_w; ++i) nnz += h_filter[i] != 0.f;
   std::vector<tetris_tile> ranked;
-  int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked);
+  int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked, (double)nnz / (double)n_w);
   if (rc) return rc;
   if (max_candidates == 0) max_candidates = 24;
   if (max_candidates < 0) max_candidates = (int)ranked.size();  // exhaustive, like the reference's table walk

@@ -227,7 +227,9 @@ int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, 
 // reads rows in the format of tuned_tiles.inc; choose_tile looks them up before the built-in table
 int load_tile_table(const char* path, int* rows_out);
 // every tile shape the kernel can run for the layer, cheapest first by the selector's time model
-int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked);
+// (density: fraction of non-zero weights when the caller knows the filter, else 0)
+int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked,
+               double density = 0.0);
 
 // output-channel order (a permutation of 0..K-1) that balances the waves of a workgroup for tile `t`
 int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_tile& t, int32_t* order);

@@ -31,6 +31,23 @@ unsigned options() {
 }
 void set_options(unsigned flags) { g_options.store(flags & 0xffffu); }
 
+// Compute units of the current device (256 on MI355X), asked once; 256 when no device can be asked (packing and
+// tile selection also run on machines without a GPU).
+int cu_count() {
+  static std::atomic<int> cached{0};
+  int v = cached.load();
+  if (v == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        n <= 0) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    cached.store(v = n);
+  }
+  return v;
+}
+
 namespace {
 
 struct Shape {
@@ -127,7 +144,7 @@ static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Ge
     return fail(TETRIS_EINVAL, "images too large for the 2 GB window of a workgroup");
   if ((long long)g.N * p->K * hw >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
   const bool four = t.waves == 16 || g.buf_bytes == kFlatHalfBufBytes;
-  const long long room = 256ll * (four ? 16 : 8);
+  const long long room = (long long)cu_count() * (four ? 16 : 8);
   const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
   g.csplit = 1;
   while (g.csplit < kMaxSplit && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
@@ -223,7 +240,7 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     // Small feature maps leave most of the 256 CUs without a workgroup: then several workgroups share an output
     // tile, each reducing a slice of the input-channel stages (at least four stages each, at most eight slices).
     const bool four = t.waves == 16 || g.buf_bytes == kHalfBufBytes;  // waves per SIMD the kernel variant allows
-    const long long room = 256ll * (g.ver == 3 && four ? 16 : 8);
+    const long long room = (long long)cu_count() * (g.ver == 3 && four ? 16 : 8);
     const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
     g.csplit = 1;
     while (g.csplit < kMaxSplit && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
@@ -305,7 +322,8 @@ static int max_tile_ic(const Shape& s, int nq, int g, int waves, int stride, int
   return best;
 }
 
-int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked) {
+int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked,
+               double density) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad layer shape");
   const bool pointwise = ks == 1 && stride == 1 && pad == 0;  // what the flat tiles take
@@ -323,7 +341,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
   //   workgroup wait for the slowest one at every stage; a CU holds eight waves.
   static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}, {2, 4}, {1, 4}};
   static const int kWaves[] = {16, 8, 4, 2, 1};
-  const double density = 0.15;  // the mask is not known here; typical of the pruned layers this runs
+  if (!(density > 0.0) || density > 1.0) density = 0.15;  // mask unknown: typical of the pruned layers this runs
   std::vector<std::pair<double, tetris_tile>> scored;
   for (int lw = 1; lw <= 62; ++lw) {
     if (lw > OW && lw > 1) break;  // wider than four images side by side could use
@@ -355,7 +373,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
         const double per_entry = four ? 40.0 + 70.0 * nq : 35.0 + 41.0 * nq;
         const double per_wave = stages * ((entries + straggle) * per_entry + 2000.0 + 60.0 * items);
         const double waves_total = (double)ugroups * kblocks * waves;
-        const double rounds = waves_total / (256.0 * (four ? 16.0 : 8.0));
+        const double rounds = waves_total / ((double)cu_count() * (four ? 16.0 : 8.0));
         // input re-read by every channel block, in units of the per-wave cycle count (a weak tie-breaker)
         const double reread = 1.0 + 0.02 * kblocks;
         const double cost = per_wave * std::max(rounds, 0.62) * reread;
@@ -389,7 +407,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
             const double entries = std::ceil((g * t * density + 0.5) / 8.0) * 8.0;
             const double per_entry = four ? 40.0 + 70.0 * nq : 35.0 + 41.0 * nq;
             const double per_wave = stages * (entries * per_entry + 600.0 + 900.0) + 6000.0;
-            const double rounds = (double)ugroups * kblocks * waves / (256.0 * (four ? 16.0 : 8.0));
+            const double rounds = (double)ugroups * kblocks * waves / ((double)cu_count() * (four ? 16.0 : 8.0));
             const double cost = per_wave * std::max(rounds, 0.62) * (1.0 + 0.02 * kblocks);
             tetris_tile tt{};
             tt.lanes_w = kFlatLanes; tt.quads = nq; tt.oc_per_wave = g; tt.waves = waves; tt.tile_ic = t;
@@ -507,8 +525,14 @@ int choose_tile(int N, int H, int W, int C, int K, int ks, int stride, int pad, 
   std::vector<tetris_tile> ranked;
   const int rc = rank_tiles(N, H, W, C, K, ks, stride, pad, &ranked);
   if (rc) return rc;
-  *t = ranked[0];
-  return TETRIS_OK;
+  for (const tetris_tile& cand : ranked) {  // the model ranks shapes the kernel's own checks may still refuse
+    Tuned e{N, H, W, C, K, ks, stride, pad, cand};
+    if (usable(e)) {
+      *t = cand;
+      return TETRIS_OK;
+    }
+  }
+  return fail(TETRIS_EINVAL, "no tile shape the kernel accepts for this layer");
 }
 
 // Output-channel order that evens out the work inside a workgroup.  A wave walks the entries of its
