@@ -5,10 +5,13 @@ A "step" is one pass of the hot path over one synthetic batch: every conv layer 
 (default: the VGG19-shaped stack at batch 16) launched once, back to back on one stream, inputs and
 packed weights already resident in HBM.  Prints ONE JSON line: whole-step dense-equivalent GFLOP/s
 (the reference's "FLOPS" figure, Tetris/spconv2d.cc:358, in decimal giga), per-layer microseconds and
-roofline fractions, the roofline of the conv kernel, and a CPU baseline measured on this box's cores.
+roofline fractions, the roofline of the conv kernel, a CPU baseline measured on this box's cores, and a
+`suites` block with the same figures for the other workloads of the metric (the single layer at batch 1,
+VGG19 at batch 1/4/8, ResNet-50, MobileNet and YOLOv3 at batch 16).  Every layer of every timed workload
+is compared with the CPU oracle on the whole batch; a mismatch beyond 1e-4 makes the exit status non-zero.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--suite vgg19|resnet50|mobilenet|yolov3|single]
-                  [--batch N] [--no-cpu] [--no-check]
+                  [--batch N] [--no-cpu] [--no-check] [--no-suites]
 """
 import argparse
 import json
@@ -23,10 +26,143 @@ sys.path.insert(0, os.path.join(ROOT, "oracle"))
 PEAK_HBM_GBS = 8000.0        # MI355X published HBM3E bandwidth
 PEAK_FP32_TFLOPS = 157.3     # MI355X published vector/matrix fp32 peak
 
-# HBM bytes per layer launch (spconv2d_kernel plus, for split layers, reduce_kernel; average over a step) from
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file, scaled by the same counters on a copy kernel of
-# known size; see profiles/.  None for workloads that were not measured.
-MEASURED_TRAFFIC_BYTES = {"vgg19/16": 1.478e8, "mobilenet/16": 4.016e7, "resnet50/16": 5.056e7}
+
+OTHER_WORKLOADS = [("single", 1), ("vgg19", 1), ("vgg19", 4), ("vgg19", 8), ("resnet50", 16), ("mobilenet", 16),
+                   ("yolov3", 16)]
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+CSRC = os.path.join(ROOT, "tetris-artifact-evalution_amd", "csrc")
+
+
+def csrc_digest():
+    """Short digest of the kernel sources, to tell whether a recorded counter figure was taken on this code."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h", ".inc", ".cpp")):
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(workload):
+    """HBM bytes per layer launch (conv kernel plus, for split layers, the reduce kernel; average over a step) from the
+    rocprofv3 FETCH_SIZE / WRITE_SIZE summaries: one text line per workload, stamped with the commit and the digest of
+    the kernel sources it was measured on.  None for a workload without a line."""
+    try:
+        lines = open(TRAFFIC_FILE).read().splitlines()
+    except OSError:
+        return None
+    for ln in lines:
+        f = ln.split()
+        if len(f) >= 6 and f[0] == workload:
+            return {"bytes_per_launch": float(f[1]) + float(f[2]), "read": float(f[1]), "written": float(f[2]),
+                    "commit": f[3], "csrc_digest": f[4], "measured": f[5], "file": "profiles/hbm_traffic.txt",
+                    "stale": f[4] != csrc_digest()}
+    return None
+
+
+def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat, masks=None, loaded=None, keep=False):
+    """Pack, time and check one (suite, batch): K steps of every layer back to back on the null stream, a per-layer
+    table, and every layer's output compared with the CPU oracle's packed-format convolution of the same tensors."""
+    dev = torch.device("cuda:0")
+    layers = W.pruned_suite(masks) if masks else W.SUITES[suite]()
+    if masks:
+        suite = layers[0].suite
+    if loaded is not None and (loaded["suite"], loaded["batch"], len(loaded["tiles"])) != (suite, N, len(layers)):
+        sys.exit("bench.py: %s was written for another workload" % args.load_tiles)
+    packs, tiles, xs, ys, works, ws = [], [], [], [], [], []
+    t_pack = 0.0
+    for li, L in enumerate(layers):
+        w = W.make_weights(L)
+        if loaded is not None:
+            tile = T.Tile(*loaded["tiles"][li])
+        elif args.tile == "autotune":
+            tile, _ = T.tile_autotune(w, N, L.H, L.W, L.stride, L.pad, args.candidates)
+        else:
+            tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+        t0 = time.perf_counter()
+        pk = T.G950Filter.for_tile(w, tile, oc_order=args.oc_order)
+        torch.cuda.synchronize()
+        t_pack += time.perf_counter() - t0
+        x = torch.from_numpy(W.make_activations(L, N)).to(dev)
+        oh, ow = W.out_hw(L)
+        y = torch.full((N, L.K, oh, ow), float("nan"), dtype=torch.float32, device=dev)
+        packs.append(pk); tiles.append(tile); xs.append(x); ys.append(y); works.append(W.work(L, N)); ws.append(w)
+    torch.cuda.synchronize()
+    if keep and args.save_tiles:
+        with open(args.save_tiles, "w") as f:
+            json.dump({"suite": suite, "batch": N,
+                       "tiles": [[t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic] for t in tiles]}, f)
+
+    def step():
+        for L, pk, tile, x, y in zip(layers, packs, tiles, xs, ys):
+            pk.launch(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
+
+    for _ in range(warmup):
+        step()
+    # The launches go to the null stream, which is torch's current stream here, so torch's events bracket them.
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+    ms_per_step_dev = ev0.elapsed_time(ev1) / steps  # device-side span of the same K steps
+
+    # every layer of the timed stack, whole batch, against the CPU oracle (not timed); the outputs started as NaN
+    check = None
+    if not args.no_check:
+        threads = min(16, O.max_threads())
+        worst, bad = (0.0, None), []
+        for L, w, x, y in zip(layers, ws, xs, ys):
+            ref = O.G950Pack(w, 32, 8).conv(x.cpu().numpy(), L.stride, L.pad, threads=threads)
+            got = y.cpu().numpy()
+            floor = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))  # same measure as tests/helpers.max_rel_err
+            err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+            if not err <= 1e-4:  # also catches NaN
+                bad.append(L.name)
+            if err > worst[0] or err != err:
+                worst = (err, L.name)
+        check = {"ok": not bad, "layers_checked": len(layers), "of": len(layers), "batch_checked": N,
+                 "max_rel_err": worst[0], "worst_layer": worst[1], "tolerance": 1e-4, "failed_layers": bad,
+                 "against": "CPU oracle, packed-format convolution of the same seeded tensors"}
+
+    # per-layer table: events on the launch stream around back-to-back launches (reference protocol,
+    # Tetris/spconv2d.cc:44-68, with fewer repetitions so the default run stays short)
+    table, t_layers = [], 0.0
+    for L, pk, tile, x, y, wk in zip(layers, packs, tiles, xs, ys, works):
+        if layer_repeat <= 0:
+            break
+        ms = pk.time(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile, warm=5, repeat=layer_repeat)
+        t = ms * 1e-3
+        t_layers += t
+        table.append({"layer": L.name, "us": round(ms * 1e3, 2),
+                      "gflops_dense_equiv": round(wk["flops_dense"] / t / 1e9, 1),
+                      "bound": wk["bound"], "roofline_frac": round(wk["t_roof"] / t, 4),
+                      "tile": [tile.lanes_w, tile.quads, tile.oc_per_wave, tile.waves, tile.tile_ic]})
+    for pk in packs:
+        pk.close()
+    fl_dense = sum(w["flops_dense"] for w in works)
+    fl_sparse = sum(w["flops_sparse"] for w in works)
+    bytes_alg = sum(w["bytes"] for w in works)
+    t_step = ms_per_step_dev * 1e-3
+    t_hbm, t_fp32 = bytes_alg / (PEAK_HBM_GBS * 1e9), fl_sparse / (PEAK_FP32_TFLOPS * 1e12)
+    out = {"suite": suite, "batch": N, "layers_per_step": len(layers), "steps": steps, "warmup": warmup,
+           "ms_per_step": round(ms_per_step, 4), "ms_per_step_device": round(ms_per_step_dev, 4),
+           "gflops_dense_equiv": round(fl_dense / (ms_per_step * 1e-3) / 1e9, 1),
+           "bound": "valu_fp32" if t_fp32 >= t_hbm else "hbm",
+           "roofline_frac": round(max(t_hbm, t_fp32) / t_step, 4),
+           "sum_of_layer_roofs_frac": round(sum(w["t_roof"] for w in works) / t_step, 4),
+           "algorithmic_bytes_per_launch": bytes_alg / len(layers),
+           "sum_layer_us": round(t_layers * 1e6, 1) if table else None,
+           "min_layer_roofline_frac": min((r["roofline_frac"] for r in table), default=None),
+           "pack_ms_total": round(t_pack * 1e3, 2), "check": check, "layers": table}
+    if keep:
+        out.update({"_layers": layers, "_xs": xs, "_ys": ys, "_works": works})
+    return out
 
 
 def main():
@@ -38,10 +174,13 @@ def main():
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--masks", metavar="NPZ", help="run the layers of a pruned network instead of --suite: a mask file "
                     "as tests/golden/masks_*.npz (zero patterns of shipped pruned weight files, seeded values)")
-    ap.add_argument("--oc-order", choices=("balanced", "file"), default="balanced",
-                    help="output-channel order of the packs: balanced over the waves of a workgroup, or as in the filter")
+    ap.add_argument("--oc-order", choices=("balanced", "file", "reference"), default="balanced",
+                    help="output-channel order of the packs: balanced over the waves of a workgroup, as in the filter, or "
+                         "the order of the reference's ReorderOutChannel pass")
+    ap.add_argument("--no-suites", action="store_true",
+                    help="time only --suite at --batch, not the other workloads of the `suites` block")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-check", action="store_true", help="skip the spot check against the oracle")
+    ap.add_argument("--no-check", action="store_true", help="skip the check of every layer against the CPU oracle")
     ap.add_argument("--layer-repeat", type=int, default=30, help="timed launches per layer for the per-layer table")
     ap.add_argument("--tile", choices=("autotune", "select"), default="select",
                     help="select: the library's own choice (its built-in table of tiles measured on MI355X, else its cycle "
@@ -85,83 +224,20 @@ def main():
         print(json.dumps({"calibrate_copy_mib": args.calibrate_copy, "dispatches": 4,
                           "bytes_read_per_dispatch": 4 * n, "bytes_written_per_dispatch": 4 * n}))
         return
-    layers = W.pruned_suite(args.masks) if args.masks else W.SUITES[args.suite]()
+    T.G950Filter(np.ones((8, 8, 1, 1), np.float32), 8, 8).close()  # loads the device code, so pack times exclude it
+    O = None
+    if not (args.no_check and args.no_cpu):
+        import oracle_py as O
+    loaded = json.load(open(args.load_tiles)) if args.load_tiles else None
+    main_run = run_workload(T, W, torch, np, O, args, args.suite, args.batch, args.steps, args.warmup, args.layer_repeat,
+                            masks=args.masks, loaded=loaded, keep=True)
+    layers, N = main_run.pop("_layers"), args.batch
+    xs, ys, works = main_run.pop("_xs"), main_run.pop("_ys"), main_run.pop("_works")
     if args.masks:
         args.suite = layers[0].suite
-    N = args.batch
-
-    packs, tiles, xs, ys, works = [], [], [], [], []
-    t_pack = 0.0
-    T.G950Filter(np.ones((8, 8, 1, 1), np.float32), 8, 8).close()  # loads the device code, so pack times exclude it
-    loaded = json.load(open(args.load_tiles)) if args.load_tiles else None
-    if loaded is not None and (loaded["suite"], loaded["batch"], len(loaded["tiles"])) != (args.suite, N, len(layers)):
-        sys.exit("bench.py: %s was written for another workload" % args.load_tiles)
-    for li, L in enumerate(layers):
-        w = W.make_weights(L)
-        if loaded is not None:
-            tile = T.Tile(*loaded["tiles"][li])
-        elif args.tile == "autotune":
-            tile, _ = T.tile_autotune(w, N, L.H, L.W, L.stride, L.pad, args.candidates)
-        else:
-            tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
-        t0 = time.perf_counter()
-        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced" if args.oc_order == "balanced" else None)
-        torch.cuda.synchronize()
-        t_pack += time.perf_counter() - t0
-        x = torch.from_numpy(W.make_activations(L, N)).to(dev)
-        oh, ow = W.out_hw(L)
-        y = torch.empty((N, L.K, oh, ow), dtype=torch.float32, device=dev)
-        packs.append(pk); tiles.append(tile); xs.append(x); ys.append(y); works.append(W.work(L, N))
-    torch.cuda.synchronize()
-    if args.save_tiles:
-        with open(args.save_tiles, "w") as f:
-            json.dump({"suite": args.suite, "batch": N,
-                       "tiles": [[t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic] for t in tiles]}, f)
-
-    def step():
-        for L, pk, tile, x, y in zip(layers, packs, tiles, xs, ys):
-            pk.launch(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
-
-    for _ in range(args.warmup):
-        step()
-    # The launches go to the null stream, which is torch's current stream here, so torch's events bracket them.
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms_per_step_dev = ev0.elapsed_time(ev1) / args.steps  # device-side span of the same K steps
-
-    # spot check of one mid-sized layer against the CPU oracle (not timed)
-    check = None
-    if not args.no_check:
-        import oracle_py as O
-        idx = min(range(len(layers)), key=lambda i: works[i]["flops_dense"] if layers[i].C > 3 else float("inf"))
-        L = layers[idx]
-        ref = O.host_conv2d(xs[idx][:1].cpu().numpy(), W.make_weights(L), L.stride, L.pad, threads=O.max_threads())
-        got = ys[idx][:1].cpu().numpy()
-        floor = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))  # same measure as tests/helpers.max_rel_err
-        err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
-        check = {"layer": L.name, "max_rel_err": err, "tolerance": 1e-4, "ok": bool(err <= 1e-4)}
-
-    # per-layer table: events on the launch stream around back-to-back launches (reference protocol,
-    # Tetris/spconv2d.cc:44-68, with fewer repetitions so the default run stays short)
-    table = []
-    t_layers = 0.0
-    for L, pk, tile, x, y, wk in zip(layers, packs, tiles, xs, ys, works):
-        if args.layer_repeat <= 0:
-            break
-        ms = pk.time(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile, warm=5, repeat=args.layer_repeat)
-        t = ms * 1e-3
-        t_layers += t
-        table.append({"layer": L.name, "us": round(ms * 1e3, 2),
-                      "gflops_dense_equiv": round(wk["flops_dense"] / t / 1e9, 1),
-                      "bound": wk["bound"], "roofline_frac": round(wk["t_roof"] / t, 4),
-                      "tile": [tile.lanes_w, tile.quads, tile.oc_per_wave, tile.waves, tile.tile_ic]})
+    ms_per_step, ms_per_step_dev, table = main_run["ms_per_step"], main_run["ms_per_step_device"], main_run["layers"]
+    check = main_run["check"]
+    failed = [] if check is None or check["ok"] else ["%s/%d" % (args.suite, N)]
 
     fl_dense = sum(w["flops_dense"] for w in works)
     fl_sparse = sum(w["flops_sparse"] for w in works)
@@ -174,7 +250,8 @@ def main():
     t_hbm, t_fp32 = bytes_alg / (PEAK_HBM_GBS * 1e9), fl_sparse / (PEAK_FP32_TFLOPS * 1e12)
     if t_fp32 >= t_hbm:
         achieved = fl_sparse / t_step / 1e12
-        roofline = {"bound": "mfma", "bound_detail": "vector fp32 FMA issued from the VALU; no MFMA is used. Peak is the "
+        roofline = {"bound": "valu_fp32", "bound_class": "mfma",
+                    "bound_detail": "compute-bound on vector fp32 FMA issued from the VALU; no MFMA is used. Peak is the "
                     "published 157.3 TFLOP/s fp32 figure, which needs packed fp32 FMA; this build compiles with packed "
                     "fp32 off, so 78.6 TFLOP/s is the most its instructions can reach",
                     "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
@@ -183,36 +260,61 @@ def main():
         achieved = bytes_alg / t_step / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(achieved / PEAK_HBM_GBS, 4)}
+    traffic = measured_traffic("%s/%d" % (args.suite, N))
     roofline.update({"kernel": "spconv2d_kernel", "launches_per_step": n_launch,
                      "avg_launch_us": round(t_step / n_launch * 1e6, 2),
                      "algorithmic_flops_per_launch": fl_sparse / n_launch,
                      "algorithmic_bytes_per_launch": bytes_alg / n_launch,
                      "sum_of_layer_roofs_frac": round(t_roof / t_step, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("%s/%d" % (args.suite, N))})
+                     "traffic": traffic["bytes_per_launch"] if traffic else None,
+                     "traffic_source": traffic})
+
+    # the other workloads of the metric ("batch 1-16" over the four suites and the single layer), each timed and
+    # checked the same way with fewer steps
+    suites = []
+    if not (args.no_suites or args.masks):
+        for suite, n in OTHER_WORKLOADS:
+            if (suite, n) == (args.suite, N):
+                continue
+            r = run_workload(T, W, torch, np, O, args, suite, n, max(5, args.steps // 2), max(3, args.warmup // 3),
+                             min(args.layer_repeat, 10))
+            t = measured_traffic("%s/%d" % (suite, n))
+            r["traffic"] = t["bytes_per_launch"] if t else None
+            if r["check"] is not None and not r["check"]["ok"]:
+                failed.append("%s/%d" % (suite, n))
+            suites.append(r)
 
     cpu = None
     if not args.no_cpu:
-        import oracle_py as O
         threads = min(O.max_threads(), 16)
-        sample_layers = layers
-        # the same workload (every layer at the benchmark's batch) once through the oracle's packed-format conv, cut
-        # short after about 25 s of wall time: a few tens of core-seconds
-        budget_s, done_fl, t_cpu, used = 25.0, 0.0, 0.0, 0
-        for L in sample_layers:
+        # The same workload (every layer at the benchmark's batch) once through the reference's own packed layout and its
+        # CPU decode -- SparseFilter arrays built with Bank-SR and ReorderOutChannel, vectorised, TILE_IC 32, walked by the
+        # restatement of HostReorderSpconv2d -- cut short after about 25 s of wall time: a few hundred core-seconds.
+        budget_s, done_fl, t_cpu, t_cpu_pack, used, agree = 25.0, 0.0, 0.0, 0.0, 0, 0.0
+        for L, x, y in zip(layers, xs, ys):
             w = W.make_weights(L)
-            xn = W.make_activations(L, N)
-            pk = O.G950Pack(w, 32, 8)
+            xn = x.cpu().numpy()
             t0 = time.perf_counter()
-            pk.conv(xn, L.stride, L.pad, threads=threads)
+            pk = O.SpfPack(w, 32, apply_reorder=True, apply_vectorize=True, bank_optimize=True, reorder_out_channel=True)
+            t_cpu_pack += time.perf_counter() - t0
+            t0 = time.perf_counter()
+            ref = pk.conv(xn, L.stride, L.pad, threads=threads)
             t_cpu += time.perf_counter() - t0
             done_fl += W.work(L, N)["flops_dense"]
             used += 1
+            if not args.no_check:
+                floor = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))
+                agree = max(agree, float(np.max(np.abs(y.cpu().numpy() - ref) / np.maximum(np.abs(ref), floor))))
             if t_cpu > budget_s:
                 break
         cpu = {"value": round(done_fl / t_cpu / 1e9, 2), "unit": "GFLOP/s", "cores": threads,
-               "kind": "port", "sample": "first %d of %d %s layers at batch %d (one pass), packed-format decode conv of the "
-               "oracle (restates HostReorderSpconv2d, spconv2d_utils.h:457-493), OpenMP over (n, oc), %.1f s wall" % (
-                   used, len(sample_layers), args.suite, N, t_cpu)}
+               "kind": "port", "sample": "first %d of %d %s layers at batch %d (one pass): the reference's SparseFilter layout "
+               "(TILE_IC 32, Bank-SR + ReorderOutChannel, 4-wide) decoded on the CPU by the oracle's restatement of "
+               "HostReorderSpconv2d (spconv2d_utils.h:457-493), OpenMP over (n, oc), %.1f s wall; packing those filters took "
+               "%.1f s more (not in the rate)" % (used, len(layers), args.suite, N, t_cpu, t_cpu_pack),
+               "gpu_vs_this_cpu_output_max_rel_err": None if args.no_check else agree}
+        if not args.no_check and not agree <= 1e-4:
+            failed.append("%s/%d vs reference-layout CPU decode" % (args.suite, N))
         # the dense CPU convolution of the same path (restates HostConv2d, tensor_utils.cc:136-170), OpenMP over (n, oc)
         L = W.single_layer()[0]
         w1, x4 = W.make_weights(L), W.make_activations(L, 4)
@@ -291,6 +393,7 @@ def main():
         "metric": "effective GFLOP/s (dense-equivalent) over the layer stack; per-layer us and roofline in `layers`",
         "value": round(fl_dense / (ms_per_step * 1e-3) / 1e9, 1),
         "unit": "GFLOP/s",
+        "check": dict(check or {}, all_workloads_ok=not failed, failed_workloads=failed) if not args.no_check else None,
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "ms_per_step_device": round(ms_per_step_dev, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
@@ -300,17 +403,21 @@ def main():
                    "tensor_seed": "base_seed ^ crc32('<suite>/<layer index>/<w|x>'), splitmix64 streams "
                                   "(tetris_amd/workloads.py)"},
         "sparse_gflops": round(fl_sparse / (ms_per_step * 1e-3) / 1e9, 1),
-        "sum_layer_us": round(t_layers * 1e6, 1) if table else None,
-        "pack_ms_total": round(t_pack * 1e3, 2),
+        "sum_layer_us": main_run["sum_layer_us"],
+        "min_layer_roofline_frac": main_run["min_layer_roofline_frac"],
+        "pack_ms_total": main_run["pack_ms_total"],
         "tile_selection": args.tile,
         "oc_order": args.oc_order,
+        "csrc_digest": csrc_digest(),
         "roofline": roofline,
         "cpu_baseline": cpu,
-        "check": check,
         "context": context,
         "layers": table,
+        "suites": suites,
     }
     print(json.dumps(out))
+    if failed:
+        sys.exit("bench.py: outputs differ from the CPU oracle beyond 1e-4 on: %s" % ", ".join(failed))
 
 
 if __name__ == "__main__":

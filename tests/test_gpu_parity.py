@@ -459,6 +459,32 @@ def test_pruned_networks_in_balanced_channel_order(env, masks):
         pk.close()
 
 
+@pytest.mark.parametrize("order", ["file", "reference", "balanced"])
+def test_channel_order_switch(env, order):
+    # The three output-channel orders a pack can be built with: as in the filter, the reference's
+    # ReorderOutChannel order (must equal the oracle's restatement of that pass), and the wave-balancing one.
+    T, torch, O = env
+    rng = np.random.default_rng(77)
+    N, C, H, W, K, ks = 2, 48, 19, 23, 72, 3
+    w = rng.standard_normal((K, C, ks, ks)).astype(np.float32)
+    w *= rng.random(w.shape) < rng.uniform(0.02, 0.5, (K, 1, 1, 1))
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    tile = T.tile_select(N, H, W, C, K, ks, 1, 1)
+    pk = T.G950Filter.for_tile(w, tile, oc_order=order)
+    got_order = np.array(pk.host_arrays()["oc_order"][:K])
+    assert sorted(got_order.tolist()) == list(range(K))
+    if order == "file":
+        assert np.array_equal(got_order, np.arange(K))
+    if order == "reference":
+        ref_perm = O.SpfPack(w, tile.tile_ic, apply_reorder=True, reorder_out_channel=True).perm
+        assert np.array_equal(got_order, ref_perm)
+    y = run_conv(T, torch, pk, x, K, ks, 1, 1, tile)
+    pk.close()
+    assert max_rel_err(y, O.host_conv2d(x, w, 1, 1, threads=4)) <= TOL
+    with pytest.raises(ValueError):
+        T.G950Filter.for_tile(w, tile, oc_order="densest-first")
+
+
 def test_tile_from_a_table_loaded_at_run_time(env, tmp_path):
     T, torch, O = env
     N, C, H, W, K, ks = 3, 24, 37, 41, 40, 3

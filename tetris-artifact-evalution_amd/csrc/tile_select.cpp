@@ -339,7 +339,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
   //   FMA is what binds it) and about 0.62 of that when it has the SIMD to itself; a stage costs about 2000
   //   cycles of barriers and stream start-up plus 60 per 16-byte slot a thread stages, and the waves of a
   //   workgroup wait for the slowest one at every stage; a CU holds eight waves.
-  static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}, {2, 4}, {1, 4}};
+  static const int kQuadG[][2] = {{2, 16}, {4, 8}, {1, 32}, {2, 8}, {1, 16}, {4, 4}, {1, 8}, {2, 4}, {1, 4}, {2, 2}, {1, 2}, {4, 2}, {1, 1}};
   static const int kWaves[] = {16, 8, 4, 2, 1};
   if (!(density > 0.0) || density > 1.0) density = 0.15;  // mask unknown: typical of the pruned layers this runs
   std::vector<std::pair<double, tetris_tile>> scored;

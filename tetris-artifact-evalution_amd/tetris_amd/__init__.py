@@ -214,11 +214,17 @@ class G950Filter:
 
     @classmethod
     def for_tile(cls, filter, tile, oc_order=None, stream=0):
-        """oc_order: None (file order), an int32 permutation, or "balanced" (oc_order_balanced for this tile)."""
+        """oc_order: None or "file" (file order), an int32 permutation, "balanced" (oc_order_balanced for this tile) or
+        "reference" (the order the reference's ReorderOutChannel pass gives, spconv2d_utils.h:249-289)."""
         if isinstance(oc_order, str):
-            if oc_order != "balanced":
-                raise ValueError("oc_order: None, a permutation or 'balanced'")
-            oc_order = oc_order_balanced(filter, tile)
+            if oc_order == "balanced":
+                oc_order = oc_order_balanced(filter, tile)
+            elif oc_order == "reference":
+                oc_order = oc_order_reference(filter, tile.tile_ic)
+            elif oc_order == "file":
+                oc_order = None
+            else:
+                raise ValueError("oc_order: None, 'file', 'balanced', 'reference' or a permutation")
         return cls(filter, tile.tile_ic, tile.oc_per_wave, oc_order, stream)
 
     def __init__(self, filter, tile_ic, oc_per_wave, oc_order=None, stream=0, device_ptr=None, shape=None):
@@ -327,6 +333,16 @@ def oc_order_balanced(filter, tile):
     K, Cc, ks, _ = w.shape
     order = np.empty(K, np.int32)
     _check(_lib.tetris_oc_order_balanced(w, Cc, K, ks, C.byref(tile), order))
+    return order
+
+
+def oc_order_reference(filter, tile_ic=32):
+    """Output-channel order of the reference's ReorderOutChannel pass (spconv2d_utils.h:249-289) for this filter."""
+    w = np.ascontiguousarray(filter, np.float32)
+    K, Cc, ks, _ = w.shape
+    f = SparseFilter(w, Cc, K, ks, TILE_IC=tile_ic, apply_reorder=True, flags=REORDER_OUT_CHANNEL)
+    order = np.array(f.oc_permutation_, np.int32)
+    f.close()
     return order
 
 
