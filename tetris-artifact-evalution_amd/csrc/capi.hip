@@ -77,7 +77,8 @@ int find_plan(tetris_g950* p, int N, int H, int W, int stride, int pad, const te
   hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
     return fail(TETRIS_EINVAL, "the first launch of a shape allocates: call tetris_g950_prepare before capturing");
-  rc = g950_bind(p, plan.geom, geom_walks_pairs(plan.geom), stream, &plan.entries, &plan.grp_off, &plan.grp_pair);
+  rc = g950_bind(p, plan.geom, geom_walks_pairs(plan.geom), stream, &plan.entries, &plan.grp_off, &plan.grp_pair,
+                 &plan.geom.heads_off);
   if (rc) return rc;
   memcpy(plan.key, key, sizeof key);
   std::lock_guard<std::mutex> lock(p->mu);

@@ -114,6 +114,10 @@ struct Geom {
   // per lane when H*W is a multiple of four.
   int qi, quads_total;
   unsigned m_qi;
+  // The bound entry array ends with a copy of the first batch (eight entries) of every stream, [group][stage][8],
+  // starting at entry `heads_off` (set when the plan is made): a workgroup reads its first batch from there, at an
+  // address it knows without having read the stream's offset first.
+  int heads_off;
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan
@@ -210,7 +214,7 @@ int spf_pack_host(const float* filter, int C, int K, int ks, int tile_ic, bool a
 // spf_pack_device.hip
 // entries of the pack bound to geometry `g`; paired: rearranged into pairs and singles (kernels that walk pairs)
 int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, const int2** entries_out,
-              const int32_t** grp_off_out, const int32_t** grp_pair_out);
+              const int32_t** grp_off_out, const int32_t** grp_pair_out, int* heads_off_out);
 
 // spf_pack_device.hip: the reference layout's device arrays as the source of a convolution
 int spf_arrays_hash(const int32_t* d_offsets, int n_off, const int32_t* d_perm, int K, const int32_t* d_position,

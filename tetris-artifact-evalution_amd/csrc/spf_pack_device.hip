@@ -283,10 +283,17 @@ __global__ void fill_pad_kernel(int2* __restrict__ out, int n) {
   if (i < n) out[i] = make_int2((int)0xC0000000u, 0);
 }
 
+// heads[seg][0..7] = the eight entries at the start of stream `seg` (for an empty stream: of the stream that follows)
+__global__ __launch_bounds__(256) void heads_kernel(const int2* __restrict__ entries, const int32_t* __restrict__ grp_off,
+                                                    int2* __restrict__ heads, int nseg) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < nseg * kBatch) heads[i] = entries[grp_off[i / kBatch] + i % kBatch];
+}
+
 }  // namespace
 
 int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, const int2** entries_out,
-              const int32_t** grp_off_out, const int32_t** grp_pair_out) {
+              const int32_t** grp_off_out, const int32_t** grp_pair_out, int* heads_off_out) {
   const BoundKey key{g.plane, g.pitch, g.par, g.stride, g.nq, paired ? 1 : 0};
   const int nseg = p->groups * p->stages;
   std::lock_guard<std::mutex> lock(p->mu);
@@ -331,7 +338,8 @@ int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, co
   if (it == p->bound.end()) {
     int2* d = nullptr;
     const long long n = (paired ? p->n_paired_entries : p->n_entries) + kBatch;  // a spare batch for the look-ahead fetch
-    TETRIS_HIP(hipMalloc(&d, sizeof(int2) * (size_t)n));
+    if (n + (long long)nseg * kBatch > 0x7fffffffll) return fail(TETRIS_EINVAL, "pack too large to bind");
+    TETRIS_HIP(hipMalloc(&d, sizeof(int2) * (size_t)(n + (long long)nseg * kBatch)));  // entries, then the streams' heads
     if (paired) {
       hipLaunchKernelGGL(bind_pairs_kernel, dim3(blocks), dim3(256), 0, stream, p->d_position, p->d_values, p->d_grp_off,
                          p->d_grp_nnz, p->d_pgrp_off, p->d_pgrp_pair, d, nseg, g.plane, g.pitch, g.par, g.stride, g.nq);
@@ -340,6 +348,9 @@ int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, co
       hipLaunchKernelGGL(bind_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p->d_position, p->d_values,
                          d, n, g.plane, g.pitch, g.par, g.stride, g.nq);
     }
+    if (nseg > 0)
+      hipLaunchKernelGGL(heads_kernel, dim3((unsigned)((nseg * kBatch + 255) / 256)), dim3(256), 0, stream, d,
+                         paired ? p->d_pgrp_off : p->d_grp_off, d + n, nseg);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       (void)hipFree(d);
@@ -350,6 +361,7 @@ int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, co
   *entries_out = it->second;
   *grp_off_out = paired ? p->d_pgrp_off : p->d_grp_off;
   *grp_pair_out = paired ? p->d_pgrp_pair : p->d_zero_pair;
+  *heads_off_out = (int)((paired ? p->n_paired_entries : p->n_entries) + kBatch);
   return TETRIS_OK;
 }
 
