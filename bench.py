@@ -165,6 +165,89 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
     return out
 
 
+def run_chain(T, W, torch, np, O, args, N, steps, warmup):
+    """The VGG19-shaped stack as a network: every convolution reads the activation of the layer before -- ReLU, and
+    2x2 max-pooling where the next layer's image is half as large (tetris_relu_maxpool) -- instead of its own synthetic
+    tensor.  Only the first layer's input is synthetic.  Timed like the stack; the last activation and every layer's
+    input are checked against the same chain on the CPU (oracle convolutions, numpy ReLU and pooling)."""
+    dev = torch.device("cuda:0")
+    layers = W.SUITES["vgg19"]()
+    packs, tiles, ws, convs, acts, pools = [], [], [], [], [], []
+    x0 = torch.from_numpy(W.make_activations(layers[0], N)).to(dev)
+    for li, L in enumerate(layers):
+        w = W.make_weights(L)
+        tile = T.tile_select(N, L.H, L.W, L.C, L.K, L.ks, L.stride, L.pad)
+        packs.append(T.G950Filter.for_tile(w, tile, oc_order=args.oc_order)); tiles.append(tile); ws.append(w)
+        pool = 2 if (li + 1 == len(layers) or layers[li + 1].H * 2 == L.H) else 1
+        pools.append(pool)
+        convs.append(torch.empty((N, L.K, L.H, L.W), dtype=torch.float32, device=dev))
+        acts.append(torch.full((N, L.K, L.H // pool, L.W // pool), float("nan"), dtype=torch.float32, device=dev))
+
+    def step():
+        x = x0
+        for L, pk, tile, y, a, pool in zip(layers, packs, tiles, convs, acts, pools):
+            pk.launch(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
+            T.relu_maxpool(y.data_ptr(), a.data_ptr(), N, L.K, L.H, L.W, pool)
+            x = a
+
+    for _ in range(warmup):
+        step()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    out = {"workload": "vgg19-shaped network pass, batch %d: 16 sparse convolutions, each followed by ReLU (2x2 max-pooling "
+           "after layers 1, 3, 7, 11 and 15); every layer's input is the previous activation" % N,
+           "ms_per_pass": round(ms, 4), "steps": steps, "warmup": warmup, "launches_per_pass": 2 * len(layers),
+           "gflops_dense_equiv": round(sum(W.work(L, N)["flops_dense"] for L in layers) / (ms * 1e-3) / 1e9, 1)}
+    if not args.no_check:
+        threads = min(16, O.max_threads())
+        ref, worst, bad = x0.cpu().numpy(), (0.0, None), []
+        for L, w, a, pool in zip(layers, ws, acts, pools):
+            ref = np.maximum(O.G950Pack(w, 32, 8).conv(np.ascontiguousarray(ref), L.stride, L.pad, threads=threads), 0.0)
+            if pool == 2:
+                n, c, h, wd = ref.shape
+                ref = ref.reshape(n, c, h // 2, 2, wd // 2, 2).max(axis=(3, 5))
+            got = a.cpu().numpy()
+            floor = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))
+            err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+            if not err <= 1e-4:
+                bad.append(L.name)
+            if err > worst[0] or err != err:
+                worst = (err, L.name)
+            ref = got  # the next layer is checked on the activation the device produced (errors do not pile up)
+        out["check"] = {"ok": not bad, "activations_checked": len(layers), "max_rel_err": worst[0], "worst_layer": worst[1],
+                        "tolerance": 1e-4, "failed_layers": bad,
+                        "against": "CPU oracle convolution + numpy ReLU / pooling of the device's previous activation"}
+    if args.dense_baseline:
+        import torch.nn.functional as F
+        wd = [torch.from_numpy(w).to(dev) for w in ws]
+
+        def dense_step():
+            x = x0
+            for L, w, pool in zip(layers, wd, pools):
+                x = F.relu(F.conv2d(x, w, None, L.stride, L.pad))
+                if pool == 2:
+                    x = F.max_pool2d(x, 2)
+
+        for _ in range(3):
+            dense_step()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            dense_step()
+        e1.record()
+        torch.cuda.synchronize()
+        out["vendor_dense_fp32_ms_per_pass"] = round(e0.elapsed_time(e1) / steps, 4)
+    for pk in packs:
+        pk.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -180,6 +263,8 @@ def main():
     ap.add_argument("--no-suites", action="store_true",
                     help="time only --suite at --batch, not the other workloads of the `suites` block")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-chain", action="store_true",
+                    help="skip the whole-network pass of the vgg19 suite (layers chained through ReLU and max-pooling)")
     ap.add_argument("--no-check", action="store_true", help="skip the check of every layer against the CPU oracle")
     ap.add_argument("--layer-repeat", type=int, default=30, help="timed launches per layer for the per-layer table")
     ap.add_argument("--tile", choices=("autotune", "select"), default="select",
@@ -283,6 +368,12 @@ def main():
             if r["check"] is not None and not r["check"]["ok"]:
                 failed.append("%s/%d" % (suite, n))
             suites.append(r)
+
+    chain = None
+    if args.suite == "vgg19" and not (args.no_chain or args.masks):
+        chain = run_chain(T, W, torch, np, O, args, N, max(5, args.steps // 2), max(3, args.warmup // 3))
+        if chain.get("check") is not None and not chain["check"]["ok"]:
+            failed.append("vgg19/%d chained" % N)
 
     cpu = None
     if not args.no_cpu:
@@ -414,6 +505,7 @@ def main():
         "context": context,
         "layers": table,
         "suites": suites,
+        "chain": chain,
     }
     print(json.dumps(out))
     if failed:

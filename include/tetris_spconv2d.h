@@ -133,6 +133,11 @@ int tetris_tile_table_load(const char* path, int* rows_out);
  * environment variable TETRIS_OPTIONS (a number) when it is set, else 0. */
 #define TETRIS_OPT_PAIRS 1u        /* halo'd kernels walk streams rearranged into pairs of entries that share one LDS read, then singles */
 #define TETRIS_OPT_NO_BANK_RULE 2u /* LDS rows packed densely: the lane-row pitch rule that keeps 16-byte LDS reads conflict-free is off */
+/* tetris_spconv2d_time and tetris_tile_autotune evict the caches (a pass over a 512 MiB buffer the library keeps until
+ * the process ends) before every timed launch and time the launches one by one.  A layer in the middle of a network
+ * finds its input, its weights and its code in HBM, and the tile that wins from warm caches, as back-to-back launches
+ * of one layer measure it (the reference's protocol, Tetris/spconv2d.cc:44-68), is not always the one that wins there. */
+#define TETRIS_OPT_COLD_TIMING 4u
 int tetris_options_set(unsigned flags);
 unsigned tetris_options_get(void);
 
@@ -257,6 +262,16 @@ int tetris_spconv2d_spf_host(const float* h_input, const float* h_filter, float*
 int tetris_spconv2d_time(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
                          int stride, int padding, const tetris_tile* tile, void* stream, int warm, int repeat,
                          float* ms_out);
+
+/* ------------------------------------------------------------------------------------------------
+ * Glue for running a stack of layers as a whole network: d_output = max(d_input, 0) (pool = 1), or that followed by
+ * 2x2 max-pooling of stride 2 (pool = 2; output img_h/2 x img_w/2 per plane, an odd last row or column is dropped).
+ * NCHW fp32 on the device, asynchronous on `stream`; pool = 1 may run in place.  No counterpart in the reference,
+ * whose mains time single layers on random inputs (Tetris/spconv2d.cc:369-450); it plays the part of the
+ * activation and pooling layers that sit between the convolutions of the networks its weight files come from.
+ * ---------------------------------------------------------------------------------------------- */
+int tetris_relu_maxpool(const float* d_input, float* d_output, int batch, int channels, int img_h, int img_w, int pool,
+                        void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Utilities of the path.

@@ -1,0 +1,123 @@
+"""Layers run as a network: ReLU / 2x2 max-pooling glue (tetris_relu_maxpool) and a chain of sparse convolutions
+whose inputs are the activations of the layer before, against numpy and the CPU oracle's dense convolution."""
+import numpy as np
+import pytest
+
+from helpers import max_rel_err, sparse_filter
+
+pytestmark = pytest.mark.gpu
+
+
+def _np_relu_pool(x, pool):
+    y = np.maximum(x, 0.0)
+    if pool == 2:
+        n, c, h, w = y.shape
+        y = y[:, :, : h // 2 * 2, : w // 2 * 2].reshape(n, c, h // 2, 2, w // 2, 2).max(axis=(3, 5))
+    return y
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 8, 8), (1, 5, 7, 9), (3, 4, 14, 14), (2, 2, 13, 16), (1, 1, 2, 2), (2, 7, 30, 20)])
+@pytest.mark.parametrize("pool", [1, 2])
+@pytest.mark.parametrize("misalign", [0, 1])
+def test_relu_maxpool_matches_numpy(shape, pool, misalign):
+    import torch
+    import tetris_amd as T
+
+    rng = np.random.default_rng(hash((shape, pool)) % 2**32)
+    x = rng.normal(size=shape).astype(np.float32)
+    n, c, h, w = shape
+    want = _np_relu_pool(x, pool)
+    # misalign: tensors that start 4 bytes into an allocation (the 16-byte paths must not be taken)
+    dx_all = torch.zeros(x.size + 4, device="cuda")
+    dy_all = torch.full((want.size + 4,), float("nan"), device="cuda")
+    dx = dx_all[misalign: misalign + x.size]
+    dy = dy_all[misalign: misalign + want.size]
+    dx.copy_(torch.from_numpy(x.reshape(-1)))
+    T.relu_maxpool(dx.data_ptr(), dy.data_ptr(), n, c, h, w, pool)
+    torch.cuda.synchronize()
+    got = dy.cpu().numpy().reshape(want.shape)
+    assert np.array_equal(got, want)
+    assert np.isnan(dy_all[misalign + want.size:].cpu().numpy()).all()  # nothing written past the end
+    if pool == 1:  # in place
+        T.relu_maxpool(dx.data_ptr(), dx.data_ptr(), n, c, h, w, 1)
+        torch.cuda.synchronize()
+        assert np.array_equal(dx.cpu().numpy().reshape(shape), want)
+
+
+def test_relu_maxpool_rejects_bad_arguments():
+    import torch
+    import tetris_amd as T
+
+    d = torch.zeros(16, device="cuda")
+    with pytest.raises(T.TetrisError):
+        T.relu_maxpool(d.data_ptr(), d.data_ptr(), 1, 1, 4, 4, 3)
+    with pytest.raises(T.TetrisError):
+        T.relu_maxpool(0, d.data_ptr(), 1, 1, 4, 4, 1)
+    with pytest.raises(T.TetrisError):
+        T.relu_maxpool(d.data_ptr(), d.data_ptr(), 1, 1, 1, 4, 2)
+
+
+def test_chain_of_layers_matches_the_oracle(oracle):
+    """conv -> ReLU -> conv -> ReLU + pool -> conv -> ReLU -> conv (1x1) on the device, every conv through the C ABI with
+    the library's tile and balanced channel order; the CPU chain uses the oracle's dense convolution."""
+    import torch
+    import tetris_amd as T
+
+    rng = np.random.default_rng(4242)
+    N, hw = 3, 28
+    specs = [(3, 24, 3, 1, 1, 0.5, 1), (24, 40, 3, 1, 1, 0.85, 2), (40, 64, 3, 1, 1, 0.9, 1), (64, 32, 1, 1, 0, 0.8, 0)]
+    x = rng.random((N, 3, hw, hw), dtype=np.float32)
+    ref = x
+    dev = torch.from_numpy(x).cuda()
+    h = hw
+    for (c, k, ks, stride, pad, sp, pool) in specs:
+        w = sparse_filter(rng, k, c, ks, sp)
+        tile = T.tile_select(N, h, h, c, k, ks, stride, pad)
+        pk = T.G950Filter.for_tile(w, tile, oc_order=T.oc_order_balanced(w, tile))
+        oh = (h + 2 * pad - ks) // stride + 1
+        y = torch.full((N, k, oh, oh), float("nan"), device="cuda")
+        pk.launch(dev.data_ptr(), y.data_ptr(), N, h, h, stride, pad, tile)
+        ref = oracle.host_conv2d(np.ascontiguousarray(ref), w, stride, pad)
+        if pool:
+            z = torch.full((N, k, oh // pool, oh // pool), float("nan"), device="cuda")
+            T.relu_maxpool(y.data_ptr(), z.data_ptr(), N, k, oh, oh, pool)
+            ref = _np_relu_pool(ref, pool)
+            dev, h = z, oh // pool
+        else:
+            dev, h = y, oh
+        torch.cuda.synchronize()
+        pk.close()
+        assert max_rel_err(dev.cpu().numpy(), ref) <= 1e-4  # north-star tolerance, layer after layer
+
+
+def test_cold_timing_option(oracle):
+    """TETRIS_OPT_COLD_TIMING: single launches timed after a cache-evicting pass.  A launch from cold caches is not
+    faster than back-to-back ones, the tuner still returns a tile that launches and computes the right thing, and the
+    option is switched off again afterwards."""
+    import torch
+    import tetris_amd as T
+
+    rng = np.random.default_rng(99)
+    N, C, H, K, ks = 8, 64, 28, 128, 1
+    w = sparse_filter(rng, K, C, ks, 0.8)
+    x = rng.random((N, C, H, H), dtype=np.float32)
+    dx = torch.from_numpy(x).cuda()
+    dy = torch.full((N, K, H, H), float("nan"), device="cuda")
+    tile = T.tile_select(N, H, H, C, K, ks, 1, 0)
+    pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+    warm = min(pk.time(dx.data_ptr(), dy.data_ptr(), N, H, H, 1, 0, tile, warm=5, repeat=30) for _ in range(3))
+    before = T.options_get()
+    try:
+        T.options_set(before | T.OPT_COLD_TIMING)
+        cold = min(pk.time(dx.data_ptr(), dy.data_ptr(), N, H, H, 1, 0, tile, warm=1, repeat=10) for _ in range(3))
+        tuned, ms = T.tile_autotune(w, N, H, H, 1, 0, 8)
+    finally:
+        T.options_set(before)
+    assert T.options_get() == before
+    assert cold >= 0.9 * warm and ms > 0, (cold, warm, ms)
+    pk2 = T.G950Filter.for_tile(w, tuned, oc_order="balanced")
+    pk2.launch(dx.data_ptr(), dy.data_ptr(), N, H, H, 1, 0, tuned)
+    torch.cuda.synchronize()
+    assert max_rel_err(dy.cpu().numpy(), oracle.host_conv2d(x, w, 1, 0)) <= 1e-4
+    pk.close()
+    pk2.close()

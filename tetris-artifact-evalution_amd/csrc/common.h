@@ -235,6 +235,9 @@ int load_tile_table(const char* path, int* rows_out);
 int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, std::vector<tetris_tile>* ranked,
                double density = 0.0);
 
+// peaks.hip: evicts the caches in front of HBM (a pass over a 512 MiB buffer on `stream`)
+int sweep_caches(hipStream_t stream);
+
 // output-channel order (a permutation of 0..K-1) that balances the waves of a workgroup for tile `t`
 int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_tile& t, int32_t* order);
 

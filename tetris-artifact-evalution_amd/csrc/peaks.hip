@@ -26,7 +26,34 @@ __global__ __launch_bounds__(256) void fma_kernel(float* out, int iters, float x
   if (s == 12345.678f) out[0] = s;  // keeps the loop alive, practically never true
 }
 
+__global__ __launch_bounds__(256) void sweep_kernel(float4* __restrict__ buf, long long n4) {
+  const long long step = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += step) {
+    float4 v = buf[i];
+    v.x += 1.f;
+    buf[i] = v;
+  }
+}
+
 }  // namespace
+
+// Reads and rewrites a 512 MiB buffer (made on first use, kept until the process ends): more than the caches in front
+// of HBM hold, so that whatever runs next on `stream` finds its tensors, its weights and its code in memory, as a
+// layer in the middle of a network does.
+int sweep_caches(hipStream_t stream) {
+  static float4* buf = nullptr;
+  static std::mutex mu;
+  const long long n4 = 32ll << 20;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!buf) {
+    TETRIS_HIP(hipMalloc(&buf, n4 * sizeof(float4)));
+    TETRIS_HIP(hipMemsetAsync(buf, 0, n4 * sizeof(float4), stream));
+  }
+  hipLaunchKernelGGL(sweep_kernel, dim3(8192), dim3(256), 0, stream, buf, n4);
+  TETRIS_HIP(hipGetLastError());
+  return TETRIS_OK;
+}
+
 }  // namespace tetris
 
 using namespace tetris;

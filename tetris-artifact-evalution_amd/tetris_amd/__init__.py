@@ -46,7 +46,7 @@ BANK_OPTIMIZE = 1
 REORDER_OUT_CHANNEL = 2
 
 OK, EINVAL, EHIP, EUNSUPPORTED, ENOTFOUND, EIO = range(6)
-OPT_PAIRS, OPT_NO_BANK_RULE = 1, 2  # tetris_options_set
+OPT_PAIRS, OPT_NO_BANK_RULE, OPT_COLD_TIMING = 1, 2, 4  # tetris_options_set
 
 
 class TetrisError(RuntimeError):
@@ -102,6 +102,7 @@ _lib.tetris_options_get.restype = C.c_uint
 _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
 _lib.tetris_tile_table_load.argtypes = [C.c_char_p, C.POINTER(C.c_int)]
 _lib.tetris_measure_peaks.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+_lib.tetris_relu_maxpool.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]
 _lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(Tile),
                                           np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")]
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
@@ -325,6 +326,13 @@ def measure_peaks(stream=0):
     c, f = C.c_float(), C.c_float()
     _check(_lib.tetris_measure_peaks(C.c_void_p(stream), C.byref(c), C.byref(f)))
     return float(c.value), float(f.value)
+
+
+def relu_maxpool(d_input, d_output, batch, channels, img_h, img_w, pool=1, stream=0):
+    """d_output = max(d_input, 0), followed by 2x2 max-pooling of stride 2 when pool == 2 (tetris_relu_maxpool);
+    device pointers to NCHW fp32, asynchronous on `stream`."""
+    _check(_lib.tetris_relu_maxpool(C.c_void_p(d_input), C.c_void_p(d_output), batch, channels, img_h, img_w, pool,
+                                    C.c_void_p(stream)))
 
 
 def oc_order_balanced(filter, tile):
