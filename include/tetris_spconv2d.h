@@ -168,6 +168,14 @@ int tetris_oc_order_balanced(const float* h_filter_oihw, int in_channel, int out
 int tetris_tile_autotune(const float* h_filter_oihw, int batch, int img_h, int img_w, int in_channel, int out_channel,
                          int kernel_size, int stride, int padding, int max_candidates, void* stream,
                          tetris_tile* out, float* ms_out);
+/* The same search, returning the `max_out` fastest candidates (all of them timed again with 2 + 10 launches), fastest
+ * first, with their milliseconds: what a tuner needs that wants to break near ties by something other than time --
+ * tetris_amd/tune.py takes, among the tiles within two per cent of the fastest, the one that moves the fewest HBM
+ * bytes by the FETCH_SIZE / WRITE_SIZE counters of rocprofv3.  out and ms_out (may be NULL) have room for max_out
+ * entries; *n_out (may be NULL) receives how many were written. */
+int tetris_tile_autotune_list(const float* h_filter_oihw, int batch, int img_h, int img_w, int in_channel,
+                              int out_channel, int kernel_size, int stride, int padding, int max_candidates,
+                              void* stream, tetris_tile* out, float* ms_out, int max_out, int* n_out);
 
 /* ------------------------------------------------------------------------------------------------
  * Conv launch on device tensors.  Replaces: SparseConv2d<float,int,int,KS,STRIDE,TILE_IC,TILE_H,TILE_W>

@@ -536,9 +536,10 @@ int tetris_oc_order_balanced(const float* h_filter, int C, int K, int ks, const 
   return balance_oc_order(h_filter, C, K, ks, *tile, order_out);
 }
 
-int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int K, int ks, int stride, int pad,
-                         int max_candidates, void* stream_, tetris_tile* out, float* ms_out) {
-  if (!h_filter || !out) return fail(TETRIS_EINVAL, "null argument");
+int tetris_tile_autotune_list(const float* h_filter, int N, int H, int W, int C, int K, int ks, int stride, int pad,
+                              int max_candidates, void* stream_, tetris_tile* out, float* ms_out, int max_out,
+                              int* n_out) {
+  if (!h_filter || !out || max_out < 1) return fail(TETRIS_EINVAL, "null argument");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs) return fail(TETRIS_EINVAL, "bad layer shape");
   size_t nnz = 0;
@@ -597,22 +598,30 @@ int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int 
   if (timed.empty()) return done(fail(TETRIS_EINVAL, "no tile shape could be launched for this layer"));
   std::stable_sort(timed.begin(), timed.end(),
                    [](const std::pair<float, tetris_tile>& a, const std::pair<float, tetris_tile>& b) { return a.first < b.first; });
-  float best_ms = 1e30f;
-  tetris_tile best = timed[0].second;
-  for (size_t i = 0; i < timed.size() && i < 4; ++i) {
+  const size_t again = std::min<size_t>(timed.size(), std::max(4, max_out));
+  for (size_t i = 0; i < again; ++i) {
     const tetris_tile& t = timed[i].second;
     float ms = 0;
     rc = time_launches(packs[{t.tile_ic, t.oc_per_wave, t.waves}], d_in, d_out, N, H, W, stride, pad, &t, stream, 2, 10,
                        &ms);
     if (rc) return done(rc);
-    if (ms < best_ms) {
-      best_ms = ms;
-      best = t;
-    }
+    timed[i].first = ms;
   }
-  *out = best;
-  if (ms_out) *ms_out = best_ms;
+  std::stable_sort(timed.begin(), timed.begin() + again,
+                   [](const std::pair<float, tetris_tile>& a, const std::pair<float, tetris_tile>& b) { return a.first < b.first; });
+  const int n = (int)std::min<size_t>(again, (size_t)max_out);
+  for (int i = 0; i < n; ++i) {
+    out[i] = timed[i].second;
+    if (ms_out) ms_out[i] = timed[i].first;
+  }
+  if (n_out) *n_out = n;
   return done(TETRIS_OK);
+}
+
+int tetris_tile_autotune(const float* h_filter, int N, int H, int W, int C, int K, int ks, int stride, int pad,
+                         int max_candidates, void* stream, tetris_tile* out, float* ms_out) {
+  return tetris_tile_autotune_list(h_filter, N, H, W, C, K, ks, stride, pad, max_candidates, stream, out, ms_out, 1,
+                                   nullptr);
 }
 
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,

@@ -106,6 +106,8 @@ _lib.tetris_relu_maxpool.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
 _lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(Tile),
                                           np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")]
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
+_lib.tetris_tile_autotune_list.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float),
+                                           C.c_int, C.POINTER(C.c_int)]
 _lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile),
                                                                                                 C.c_void_p]
 _lib.tetris_g950_prepare.argtypes = [C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile), C.c_void_p]
@@ -362,6 +364,18 @@ def tile_autotune(filter, batch, img_h, img_w, stride, padding, max_candidates=0
     _check(_lib.tetris_tile_autotune(w, batch, img_h, img_w, Cc, K, ks, stride, padding, max_candidates,
                                      C.c_void_p(stream), C.byref(t), C.byref(ms)))
     return t, float(ms.value)
+
+
+def tile_autotune_list(filter, batch, img_h, img_w, stride, padding, max_candidates=0, max_out=4, stream=0):
+    """-> [(Tile, ms per launch), ...]: the `max_out` fastest measured tile shapes, fastest first
+    (tetris_tile_autotune_list)."""
+    w = np.ascontiguousarray(filter, np.float32)
+    K, Cc, ks, _ = w.shape
+    tiles, ms, n = (Tile * max_out)(), (C.c_float * max_out)(), C.c_int()
+    _check(_lib.tetris_tile_autotune_list(w, batch, img_h, img_w, Cc, K, ks, stride, padding, max_candidates,
+                                          C.c_void_p(stream), tiles, ms, max_out, C.byref(n)))
+    return [(Tile(tiles[i].lanes_w, tiles[i].quads, tiles[i].oc_per_wave, tiles[i].waves, tiles[i].tile_ic), float(ms[i]))
+            for i in range(n.value)]
 
 
 def SparseConv2d(input, offsets, stage_len, oc_permutation, position, values, output, batch_size, img_h, img_w,
