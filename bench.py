@@ -116,18 +116,23 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
     check = None
     if not args.no_check:
         threads = min(16, O.max_threads())
-        worst, bad = (0.0, None), []
+        worst, bad, strict, big = (0.0, None), [], 0.0, 0.0
         for L, w, x, y in zip(layers, ws, xs, ys):
             ref = O.G950Pack(w, 32, 8).conv(x.cpu().numpy(), L.stride, L.pad, threads=threads)
             got = y.cpu().numpy()
+            diff = np.abs(got - ref)
             floor = max(1e-3, 1e-2 * float(np.max(np.abs(ref))))  # same measure as tests/helpers.max_rel_err
-            err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+            err = float(np.max(diff / np.maximum(np.abs(ref), floor)))
+            # the same errors under stricter denominators: an absolute floor of 1e-3 alone, and the largest |ref| alone
+            strict = max(strict, float(np.max(diff / np.maximum(np.abs(ref), 1e-3))))
+            big = max(big, float(np.max(diff)) / float(np.max(np.abs(ref))))
             if not err <= 1e-4:  # also catches NaN
                 bad.append(L.name)
             if err > worst[0] or err != err:
                 worst = (err, L.name)
         check = {"ok": not bad, "layers_checked": len(layers), "of": len(layers), "batch_checked": N,
                  "max_rel_err": worst[0], "worst_layer": worst[1], "tolerance": 1e-4, "failed_layers": bad,
+                 "max_rel_err_floor_1e-3_only": strict, "max_abs_err_over_max_abs_ref": big,
                  "against": "CPU oracle, packed-format convolution of the same seeded tensors"}
 
     # per-layer table: events on the launch stream around back-to-back launches (reference protocol,
