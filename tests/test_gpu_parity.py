@@ -149,6 +149,34 @@ def test_flat_tiles_of_pointwise_layers(env, tile, shape):
     assert e.value.code == T.EINVAL
 
 
+@pytest.mark.parametrize("tile", [(1, 8, 16), (2, 4, 16), (1, 2, 16), (2, 16, 8), (4, 8, 8), (1, 4, 8)])
+@pytest.mark.parametrize("shape", [(3, 12, 23, 29, 37, 2), (5, 70, 14, 14, 130, 2), (2, 33, 13, 13, 16, 2),
+                                   (4, 300, 28, 28, 24, 2), (2, 9, 20, 31, 40, 3), (9, 40, 7, 7, 64, 2)])
+def test_flat_tiles_of_strided_pointwise_layers(env, tile, shape):
+    # 1x1 layers of stride 2 or 3 (projection shortcuts): the flat tile runs on the sub-grid the layer reads; a quad is
+    # four sub-grid pixels, staged as four dwords, and may straddle two rows of the image.  Odd sizes (the sub-grid's
+    # last row and column are the image's last), quads cut short at the end of an image, split channel reduction.
+    T, torch, O = env
+    nq, g, waves = tile
+    N, C, H, W, K, stride = shape
+    rng = np.random.default_rng(nq * 1000 + g * 10 + waves + C + stride)
+    w = sparse_filter(rng, K, C, 1, 0.7)
+    x = (relu_like(rng, (N, C, H, W)) + 0.25).astype(np.float32)
+    ref = O.host_conv2d(x, w, stride, 0, threads=4)
+    ran = 0
+    for tile_ic in (3, 16, 64):
+        t = T.Tile(64, nq, g, waves, tile_ic)
+        pk = T.G950Filter(w, tile_ic, g)
+        try:
+            y = run_conv(T, torch, pk, x, K, 1, stride, 0, t)
+        except T.TetrisError as e:
+            assert e.code == T.EINVAL and "LDS" in str(e), str(e)
+            continue
+        ran += 1
+        assert max_rel_err(y, ref) <= TOL, (tile, shape, tile_ic)
+    assert ran >= 2
+
+
 @pytest.mark.parametrize("opts", [1, 2, 3])
 def test_ablation_switches_keep_the_results(env, opts):
     # TETRIS_OPT_PAIRS (streams rearranged into pairs sharing an LDS read + singles) and TETRIS_OPT_NO_BANK_RULE (LDS

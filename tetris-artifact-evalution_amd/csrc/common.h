@@ -112,8 +112,10 @@ struct Geom {
   // 1 KiB row per staged channel and unit (lane l at byte 16*l): staging is one 16-byte-per-lane load that writes LDS
   // directly per (channel, unit), reads are aligned 16-byte accesses at consecutive addresses, stores are 16 bytes
   // per lane when H*W is a multiple of four.
+  // A strided pointwise layer keeps the flat tile on the sub-grid it reads (H, W above; element (row, col) lies at
+  // row*step*in_w + col*step of a plane of in_hw floats): a lane's quad is then staged as four separate dwords.
   int qi, quads_total;
-  unsigned m_qi;
+  unsigned m_qi, m_ow;
   // The bound entry array ends with a copy of the first batch (eight entries) of every stream, [group][stage][8],
   // starting at entry `heads_off` (set when the plan is made): a workgroup reads its first batch from there, at an
   // address it knows without having read the stream's offset first.

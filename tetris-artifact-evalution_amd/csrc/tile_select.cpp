@@ -106,8 +106,8 @@ int image_stride(const Shape& s, int tile_ic, int stride) {
 
 // Geometry of a flat tile (lanes_w == 64) for a pointwise layer; `g` holds the layer and the tile's quads, slots and waves.
 static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Geom* out) {
-  if (p->ks != 1 || g.stride != 1 || g.pad != 0 || g.step != 1)
-    return fail(TETRIS_EINVAL, "flat tiles (lanes_w = %d) are for 1x1 layers of stride 1 without padding", kFlatLanes);
+  if (p->ks != 1 || g.stride != 1 || g.pad != 0 || g.step < 1)  // a strided layer arrives as stride 1 on its sub-grid
+    return fail(TETRIS_EINVAL, "flat tiles (lanes_w = %d) are for 1x1 layers without padding", kFlatLanes);
   if (t.waves != 8 && t.waves != 16) return fail(TETRIS_EINVAL, "bad tile: flat tiles take 8 or 16 waves (got %d)", t.waves);
   if (g.nq != 1 && g.nq != 2 && g.nq != 4) return fail(TETRIS_EINVAL, "bad tile: quads=%d", g.nq);
   if (t.oc_per_wave != p->g)
@@ -123,6 +123,8 @@ static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Ge
     return fail(TETRIS_EINVAL, "too many pixels for the kernel's index arithmetic");
   g.quads_total = (int)quads;
   g.m_qi = magic_reciprocal(g.qi);
+  if (hw * g.W >= (1ll << 32)) return fail(TETRIS_EINVAL, "too many pixels for the kernel's index arithmetic");
+  g.m_ow = magic_reciprocal(g.W);
   g.buf_bytes = (t.waves == 8 && g.g * 4 * g.nq <= kAccRegs / 2 && g.nq <= 2) ? kFlatHalfBufBytes : kFlatBufBytes;
   g.region = g.buf_bytes / g.nq;
   g.plane = 256; g.pitch = 0; g.par = 0; g.lw = g.lr = 64; g.lh = 1; g.thi = 1; g.nb = 1; g.ng = 64; g.ih = 1;
@@ -140,7 +142,7 @@ static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Ge
   if ((long long)g.ugroups * g.kblocks > (1ll << 28)) return fail(TETRIS_EINVAL, "grid too large");
   // a workgroup reaches its images through one 2 GB window on the input and one on the output
   const long long span = (64ll * g.nq + g.qi - 1) / g.qi + 2;  // images a workgroup's quads can touch, and a spare
-  if (4ll * hw * std::max(p->C, p->K) * span >= (1ll << 31))
+  if (4ll * std::max((long long)g.in_hw * p->C, hw * p->K) * span >= (1ll << 31))
     return fail(TETRIS_EINVAL, "images too large for the 2 GB window of a workgroup");
   if ((long long)g.N * p->K * hw >= (1ll << 40)) return fail(TETRIS_EINVAL, "output too large");
   const bool four = t.waves == 16 || g.buf_bytes == kFlatHalfBufBytes;
@@ -326,7 +328,7 @@ int rank_tiles(int N, int H, int W, int C, int K, int ks, int stride, int pad, s
                double density) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad layer shape");
-  const bool pointwise = ks == 1 && stride == 1 && pad == 0;  // what the flat tiles take
+  const bool pointwise = ks == 1 && pad == 0;  // what the flat tiles take (a strided one on the sub-grid it reads)
   if (ks == 1 && stride > 1 && pad == 0) {  // run as a stride-1 layer on the sub-grid it reads (see make_geom)
     H = (H - 1) / stride + 1;
     W = (W - 1) / stride + 1;
