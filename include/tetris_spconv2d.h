@@ -104,7 +104,10 @@ int tetris_g950_host_arrays(tetris_g950* p, tetris_g950_arrays* out);
  * ---------------------------------------------------------------------------------------------- */
 typedef struct tetris_tile {
   int32_t lanes_w;     /* active lanes across a tile row (1..62); the tile is 4*lanes_w columns wide.  A tile at
-                          least twice (four times) as wide as the output puts 2 (4) images side by side */
+                          least twice (four times) as wide as the output puts 2 (4) images side by side.
+                          64 = the flat tile of 1x1 layers without padding (any stride): a lane owns four
+                          consecutive pixels of the image (of the sub-grid a strided layer reads), 64 lanes a run of
+                          256; takes waves = 8 or 16 */
   int32_t quads;       /* 4-pixel groups per lane (1, 2 or 4)                                      */
   int32_t oc_per_wave; /* output channels a wave accumulates at once; oc_per_wave*4*quads <= 128 (64 when waves = 16) */
   int32_t waves;       /* waves per workgroup (1, 2, 4, 8 or 16); it computes waves*oc_per_wave channels */
