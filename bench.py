@@ -172,9 +172,11 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
 
 def run_chain(T, W, torch, np, O, args, N, steps, warmup):
     """The VGG19-shaped stack as a network: every convolution reads the activation of the layer before -- ReLU, and
-    2x2 max-pooling where the next layer's image is half as large (tetris_relu_maxpool) -- instead of its own synthetic
-    tensor.  Only the first layer's input is synthetic.  Timed like the stack; the last activation and every layer's
-    input are checked against the same chain on the CPU (oracle convolutions, numpy ReLU and pooling)."""
+    2x2 max-pooling where the next layer's image is half as large -- instead of its own synthetic tensor.  Only the
+    first layer's input is synthetic.  Timed like the stack, twice: with the activation applied by the layer's own
+    kernels (tetris_spconv2d_launch_act; the figure reported) and as a second pass per layer (tetris_relu_maxpool).
+    The last activation and every layer's input are checked against the same chain on the CPU (oracle convolutions,
+    numpy ReLU and pooling)."""
     dev = torch.device("cuda:0")
     layers = W.SUITES["vgg19"]()
     packs, tiles, ws, convs, acts, pools = [], [], [], [], [], []
@@ -188,26 +190,49 @@ def run_chain(T, W, torch, np, O, args, N, steps, warmup):
         convs.append(torch.empty((N, L.K, L.H, L.W), dtype=torch.float32, device=dev))
         acts.append(torch.full((N, L.K, L.H // pool, L.W // pool), float("nan"), dtype=torch.float32, device=dev))
 
-    def step():
+    fused = [pk.act_supported(N, L.H, L.W, L.stride, L.pad, tile, pool)
+             for L, pk, tile, pool in zip(layers, packs, tiles, pools)]
+
+    def step_two_pass():  # every activation as a second pass over the layer's output
         x = x0
         for L, pk, tile, y, a, pool in zip(layers, packs, tiles, convs, acts, pools):
             pk.launch(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
             T.relu_maxpool(y.data_ptr(), a.data_ptr(), N, L.K, L.H, L.W, pool)
             x = a
 
-    for _ in range(warmup):
-        step()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(steps):
-        step()
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / steps
+    def step():  # activations written by the layer's own kernels where its tile can (tetris_spconv2d_launch_act)
+        x = x0
+        for L, pk, tile, y, a, pool, f in zip(layers, packs, tiles, convs, acts, pools, fused):
+            if f:
+                pk.launch_act(x.data_ptr(), a.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile, pool)
+            else:
+                pk.launch_act(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile, T.ACT_RELU)
+                T.relu_maxpool(y.data_ptr(), a.data_ptr(), N, L.K, L.H, L.W, pool)
+            x = a
+
+    def timed(fn):
+        for _ in range(warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    ms_two = timed(step_two_pass)
+    for a in acts:
+        a.fill_(float("nan"))
+    ms = timed(step)  # last, so that the activations checked below are the fused pass's
     out = {"workload": "vgg19-shaped network pass, batch %d: 16 sparse convolutions, each followed by ReLU (2x2 max-pooling "
-           "after layers 1, 3, 7, 11 and 15); every layer's input is the previous activation" % N,
-           "ms_per_pass": round(ms, 4), "steps": steps, "warmup": warmup, "launches_per_pass": 2 * len(layers),
+           "after layers 1, 3, 7, 11 and 15); every layer's input is the previous activation; the activation is applied "
+           "by the layer's own kernels as they write (tetris_spconv2d_launch_act)" % N,
+           "ms_per_pass": round(ms, 4), "steps": steps, "warmup": warmup,
+           "launches_per_pass": len(layers) + sum(not f for f in fused),
+           "layers_with_the_activation_as_a_second_pass": [L.name for L, f in zip(layers, fused) if not f],
+           "ms_per_pass_activations_as_second_passes": round(ms_two, 4),
            "gflops_dense_equiv": round(sum(W.work(L, N)["flops_dense"] for L in layers) / (ms * 1e-3) / 1e9, 1)}
     if not args.no_check:
         threads = min(16, O.max_threads())
@@ -241,6 +266,7 @@ def run_chain(T, W, torch, np, O, args, N, steps, warmup):
 
         for _ in range(3):
             dense_step()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record()
         for _ in range(steps):

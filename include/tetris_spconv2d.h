@@ -196,6 +196,24 @@ int tetris_tile_autotune_list(const float* h_filter_oihw, int batch, int img_h, 
 int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
                            int stride, int padding, const tetris_tile* tile, void* stream);
 
+/* tetris_spconv2d_launch with the activation that follows the layer done on the way out, instead of by a second pass
+ * over the tensor (tetris_relu_maxpool): the sums never reach memory.  No counterpart in the reference, whose layers
+ * are timed one by one without activations.  TETRIS_ACT_RELU: d_output = max(conv, 0), same shape, every tile.
+ * TETRIS_ACT_RELU_POOL2: ReLU then 2x2 max-pooling of stride 2, d_output is [batch][out_channel][oh/2][ow/2] (an odd
+ * last row or column is dropped); a split layer pools in its adding kernel, any other layer inside the conv kernel,
+ * which needs a halo'd tile (not the flat tile of pointwise layers) with an even number of lanes per row and of rows
+ * per unit -- otherwise TETRIS_EUNSUPPORTED and nothing is launched (tetris_spconv2d_act_supported tells beforehand,
+ * in *supported; launch with TETRIS_ACT_RELU and pool with tetris_relu_maxpool then).  Results are
+ * bit-identical to tetris_spconv2d_launch followed by tetris_relu_maxpool.  Plans, scratch and graph capture as for
+ * tetris_spconv2d_launch. */
+#define TETRIS_ACT_NONE 0
+#define TETRIS_ACT_RELU 1
+#define TETRIS_ACT_RELU_POOL2 2
+int tetris_spconv2d_launch_act(tetris_g950* p, const float* d_input, float* d_output, int batch, int img_h, int img_w,
+                               int stride, int padding, const tetris_tile* tile, int activation, void* stream);
+int tetris_spconv2d_act_supported(tetris_g950* p, int batch, int img_h, int img_w, int stride, int padding,
+                                  const tetris_tile* tile, int activation, int* supported);
+
 /* Makes everything tetris_spconv2d_launch would otherwise make on its first call for (input shape, tile) on
  * `stream`: the launch plan, the entries bound to the tile geometry and, for a split layer, the partial-sum buffer of
  * that stream.  After it returns, launches with the same arguments allocate nothing and can be captured into a HIP

@@ -121,3 +121,69 @@ def test_cold_timing_option(oracle):
     assert max_rel_err(dy.cpu().numpy(), oracle.host_conv2d(x, w, 1, 0)) <= 1e-4
     pk.close()
     pk2.close()
+
+
+# (tile, N, C, K, H, W, ks, stride, pad, pooling expected to be possible)
+_FUSED_CASES = [
+    ((14, 2, 8, 16, 16), 4, 32, 128, 56, 56, 3, 1, 1, True),    # sixteen waves, three LDS buffers
+    ((14, 2, 8, 8, 8), 3, 16, 64, 56, 56, 3, 1, 1, True),       # eight waves
+    ((14, 1, 8, 8, 16), 3, 32, 64, 56, 56, 3, 1, 1, True),
+    ((28, 4, 8, 4, 3), 2, 3, 64, 56, 56, 3, 1, 1, True),        # single LDS tile, register staging
+    ((7, 2, 2, 16, 16), 2, 16, 32, 28, 28, 3, 1, 1, False),     # odd number of lanes per row
+    ((14, 2, 8, 16, 16), 5, 16, 128, 14, 14, 3, 1, 1, True),    # four images side by side, one stage: not split
+    ((14, 2, 8, 16, 16), 3, 16, 128, 28, 28, 3, 1, 1, True),    # two images side by side
+    ((14, 2, 8, 16, 16), 2, 256, 128, 14, 14, 3, 1, 1, True),   # split layer: the adding kernel pools (scalar path)
+    ((14, 2, 8, 16, 16), 1, 256, 128, 28, 28, 3, 1, 1, True),   # split layer, 16-byte path of the adding kernel
+    ((16, 1, 4, 8, 8), 2, 8, 24, 15, 15, 3, 1, 1, True),        # odd output: last row and column dropped
+    ((14, 1, 8, 16, 8), 2, 16, 64, 56, 56, 3, 2, 1, True),      # stride 2
+    ((13, 2, 8, 16, 8), 2, 16, 64, 52, 52, 3, 1, 1, False),
+    ((64, 1, 4, 16, 64), 2, 64, 64, 28, 28, 1, 1, 0, None),     # flat tile: pools only where the layer is split
+    ((64, 1, 4, 16, 64), 2, 512, 64, 7, 7, 1, 1, 0, None),
+]
+
+
+@pytest.mark.parametrize("case", _FUSED_CASES, ids=lambda c: "t%s_n%d_c%d_k%d_%dx%d_ks%d_s%d" % (("-".join(map(str, c[0])),) + c[1:8]))
+def test_activation_fused_into_the_launch(case, oracle):
+    """tetris_spconv2d_launch_act: ReLU, and ReLU + 2x2 max-pooling, written by the conv (or the adding) kernel itself
+    are bit-identical to the plain launch followed by tetris_relu_maxpool; the ReLU result also matches the oracle.
+    Where a tile cannot pool, the launch is refused with TETRIS_EUNSUPPORTED and writes nothing."""
+    import torch
+    import tetris_amd as T
+
+    tl, N, Cc, K, H, W, ks, stride, pad, can_pool = case
+    rng = np.random.default_rng(hash(case[:9]) % (1 << 32))
+    tile = T.Tile(*tl)
+    w = sparse_filter(rng, K, Cc, ks, 0.8)
+    x = (rng.random((N, Cc, H, W), dtype=np.float32) - 0.5)
+    OH, OW = (H + 2 * pad - ks) // stride + 1, (W + 2 * pad - ks) // stride + 1
+    pk = T.G950Filter.for_tile(w, tile, oc_order=T.oc_order_balanced(w, tile))
+    dx = torch.from_numpy(x).cuda()
+    y = torch.full((N, K, OH, OW), float("nan"), device="cuda")
+    pk.launch(dx.data_ptr(), y.data_ptr(), N, H, W, stride, pad, tile)
+    for act in (T.ACT_RELU, T.ACT_RELU_POOL2):
+        shape = (N, K, OH, OW) if act == T.ACT_RELU else (N, K, OH // 2, OW // 2)
+        two = torch.full(shape, float("nan"), device="cuda")
+        T.relu_maxpool(y.data_ptr(), two.data_ptr(), N, K, OH, OW, act)
+        one = torch.full(shape, float("nan"), device="cuda")
+        ok = pk.act_supported(N, H, W, stride, pad, tile, act)
+        if act == T.ACT_RELU:
+            assert ok
+        elif can_pool is not None:
+            assert ok == can_pool
+        if not ok:
+            with pytest.raises(T.TetrisError) as e:
+                pk.launch_act(dx.data_ptr(), one.data_ptr(), N, H, W, stride, pad, tile, act)
+            assert e.value.code == 3  # TETRIS_EUNSUPPORTED
+            torch.cuda.synchronize()
+            assert bool(torch.isnan(one).all())
+            continue
+        pk.launch_act(dx.data_ptr(), one.data_ptr(), N, H, W, stride, pad, tile, act)
+        torch.cuda.synchronize()
+        assert not bool(torch.isnan(one).any())
+        assert torch.equal(one, two)
+        if act == T.ACT_RELU:
+            ref = np.maximum(oracle.host_conv2d(x, w, stride, pad), 0.0)
+            assert max_rel_err(one.cpu().numpy(), ref) <= 1e-4
+    with pytest.raises(T.TetrisError):
+        pk.launch_act(dx.data_ptr(), y.data_ptr(), N, H, W, stride, pad, tile, 3)
+    pk.close()

@@ -117,7 +117,7 @@ int partial_buffer(tetris_g950* p, hipStream_t stream, size_t need, bool grow, f
 }
 
 int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,
-               const tetris_tile* tile, hipStream_t stream) {
+               const tetris_tile* tile, hipStream_t stream, int act = 0) {
   if (!p || !d_in || !d_out) return fail(TETRIS_EINVAL, "null argument");
   Plan plan;
   int rc = find_plan(p, N, H, W, stride, pad, tile, stream, true, &plan);
@@ -127,7 +127,8 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
     rc = partial_buffer(p, stream, partial_bytes_of(plan.geom), true, &d_partial);
     if (rc) return rc;
   }
-  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, stream);
+  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, act,
+                     stream);
 }
 
 // ---- scratch of the entry point that allocates nothing ------------------------------------------------------------
@@ -629,6 +630,26 @@ int tetris_spconv2d_launch(tetris_g950* p, const float* d_in, float* d_out, int 
   return run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, static_cast<hipStream_t>(stream));
 }
 
+int tetris_spconv2d_launch_act(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride,
+                               int pad, const tetris_tile* tile, int activation, void* stream) {
+  if (activation < TETRIS_ACT_NONE || activation > TETRIS_ACT_RELU_POOL2)
+    return fail(TETRIS_EINVAL, "unknown activation %d", activation);
+  return run_launch(p, d_in, d_out, N, H, W, stride, pad, tile, static_cast<hipStream_t>(stream), activation);
+}
+
+int tetris_spconv2d_act_supported(tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile* tile,
+                                  int activation, int* supported) {
+  if (!p || !tile || !supported) return fail(TETRIS_EINVAL, "null argument");
+  if (activation < TETRIS_ACT_NONE || activation > TETRIS_ACT_RELU_POOL2)
+    return fail(TETRIS_EINVAL, "unknown activation %d", activation);
+  Geom g;
+  const int rc = make_geom(p, N, H, W, stride, pad, *tile, &g);
+  if (rc) return rc;
+  *supported = activation != TETRIS_ACT_RELU_POOL2 ||
+               (g.OH >= 2 && g.OW >= 2 && (g.csplit > 1 || geom_pools_in_kernel(g)));
+  return TETRIS_OK;
+}
+
 int tetris_g950_prepare(tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile* tile, void* stream_) {
   if (!p) return fail(TETRIS_EINVAL, "null argument");
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -671,7 +692,8 @@ int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_in, float* d_o
   }
   // Every element of the partial sums that reduce_kernel reads is written by this launch's conv kernel first, so
   // what an earlier call left in the array needs no clearing.
-  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, stream);
+  return launch_conv(plan.geom, d_in, d_out, d_partial, plan.entries, plan.grp_off, plan.grp_pair, p->d_oc_order, 0,
+                     stream);
 }
 
 int tetris_spconv2d_launch_spf_arrays(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,

@@ -120,6 +120,9 @@ struct Geom {
   // starting at entry `heads_off` (set when the plan is made): a workgroup reads its first batch from there, at an
   // address it knows without having read the stream's offset first.
   int heads_off;
+  // What a kernel does to a finished sum before it writes it (set per launch): 0 nothing, 1 ReLU, 2 ReLU and 2x2
+  // max-pooling inside the halo'd kernels (the output tensor is then N x K x OH/2 x OW/2).
+  int act;
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan
@@ -246,8 +249,12 @@ int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_til
 // spconv2d_kernel.hip
 // launches the conv; when the geometry splits the channel reduction (csplit > 1) the workgroups write their partial
 // sums to d_partial ([csplit] outputs) and a second kernel adds the slices, in order, into d_out
+// act: 0 = d_out gets the sums; 1 = their ReLU; 2 = ReLU and 2x2 max-pooling (d_out is N x K x OH/2 x OW/2), done by
+// the adding kernel of a split layer and otherwise inside the conv kernel where geom_pools_in_kernel allows (else
+// TETRIS_EUNSUPPORTED, nothing launched)
 int launch_conv(const Geom& g, const float* d_in, float* d_out, float* d_partial, const int2* entries,
-                const int32_t* grp_off, const int32_t* grp_pair, const int32_t* oc_order, hipStream_t stream);
+                const int32_t* grp_off, const int32_t* grp_pair, const int32_t* oc_order, int act, hipStream_t stream);
+bool geom_pools_in_kernel(const Geom& g);
 // whether the kernel of geometry `g` walks paired streams
 bool geom_walks_pairs(const Geom& g);
 

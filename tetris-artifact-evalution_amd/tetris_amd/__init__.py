@@ -47,6 +47,7 @@ REORDER_OUT_CHANNEL = 2
 
 OK, EINVAL, EHIP, EUNSUPPORTED, ENOTFOUND, EIO = range(6)
 OPT_PAIRS, OPT_NO_BANK_RULE, OPT_COLD_TIMING = 1, 2, 4  # tetris_options_set
+ACT_NONE, ACT_RELU, ACT_RELU_POOL2 = 0, 1, 2  # tetris_spconv2d_launch_act
 
 
 class TetrisError(RuntimeError):
@@ -103,6 +104,10 @@ _lib.tetris_tile_select.argtypes = [C.c_int] * 8 + [C.POINTER(Tile)]
 _lib.tetris_tile_table_load.argtypes = [C.c_char_p, C.POINTER(C.c_int)]
 _lib.tetris_measure_peaks.argtypes = [C.c_void_p, C.POINTER(C.c_float), C.POINTER(C.c_float)]
 _lib.tetris_relu_maxpool.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]
+_lib.tetris_spconv2d_launch_act.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
+    C.POINTER(Tile), C.c_int, C.c_void_p]
+_lib.tetris_spconv2d_act_supported.argtypes = [C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile), C.c_int,
+                                               C.POINTER(C.c_int)]
 _lib.tetris_oc_order_balanced.argtypes = [_f32p, C.c_int, C.c_int, C.c_int, C.POINTER(Tile),
                                           np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")]
 _lib.tetris_tile_autotune.argtypes = [_f32p] + [C.c_int] * 9 + [C.c_void_p, C.POINTER(Tile), C.POINTER(C.c_float)]
@@ -262,6 +267,20 @@ class G950Filter:
         _check(_lib.tetris_spconv2d_launch(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h, img_w,
                                            stride, padding, C.byref(tile) if tile is not None else None,
                                            C.c_void_p(stream)))
+
+    def launch_act(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile, activation, stream=0):
+        """launch() with ReLU (ACT_RELU) or ReLU + 2x2 max-pooling (ACT_RELU_POOL2, output N x K x OH/2 x OW/2) done as
+        the sums are written (tetris_spconv2d_launch_act)."""
+        _check(_lib.tetris_spconv2d_launch_act(self._h, C.c_void_p(d_input), C.c_void_p(d_output), batch, img_h, img_w,
+                                               stride, padding, C.byref(tile) if tile is not None else None,
+                                               activation, C.c_void_p(stream)))
+
+    def act_supported(self, batch, img_h, img_w, stride, padding, tile, activation):
+        """Whether launch_act can do `activation` for this shape and tile (tetris_spconv2d_act_supported)."""
+        yes = C.c_int()
+        _check(_lib.tetris_spconv2d_act_supported(self._h, batch, img_h, img_w, stride, padding, C.byref(tile),
+                                                  activation, C.byref(yes)))
+        return bool(yes.value)
 
     def prepare(self, batch, img_h, img_w, stride, padding, tile=None, stream=0):
         """Makes the launch plan (and a split layer's partial-sum buffer on `stream`) ahead of the first launch."""
