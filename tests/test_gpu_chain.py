@@ -187,3 +187,55 @@ def test_activation_fused_into_the_launch(case, oracle):
     with pytest.raises(T.TetrisError):
         pk.launch_act(dx.data_ptr(), y.data_ptr(), N, H, W, stride, pad, tile, 3)
     pk.close()
+
+
+def test_chain_with_fused_activations_in_a_hip_graph(oracle):
+    """conv+ReLU -> conv+ReLU+pool -> conv+ReLU (split layer) captured once and replayed on new inputs: each replay
+    equals the eager two-pass chain bit for bit and the CPU chain within tolerance."""
+    import torch
+    import tetris_amd as T
+
+    rng = np.random.default_rng(77)
+    N, H = 4, 28
+    specs = [(8, 32, 3, 1, T.ACT_RELU), (32, 64, 3, 1, T.ACT_RELU_POOL2), (64, 256, 3, 1, T.ACT_RELU)]  # C, K, ks, pad, act
+    x0 = torch.zeros((N, 8, H, H), device="cuda")
+    layers, cur, h = [], x0, H
+    for C, K, ks, pad, act in specs:
+        w = sparse_filter(rng, K, C, ks, 0.8)
+        tile = T.tile_select(N, h, h, C, K, ks, 1, pad)
+        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+        if not pk.act_supported(N, h, h, 1, pad, tile, act):  # the table's tile for this shape cannot pool
+            tile = T.Tile(14, 2, tile.oc_per_wave, 16, tile.tile_ic)
+            assert pk.act_supported(N, h, h, 1, pad, tile, act)
+        oh = h // 2 if act == T.ACT_RELU_POOL2 else h
+        y = torch.empty((N, K, oh, oh), device="cuda")
+        raw = torch.empty((N, K, h, h), device="cuda")
+        layers.append((w, pk, tile, cur, y, raw, h, pad, act))
+        cur, h = y, oh
+
+    side = torch.cuda.Stream()
+    for _, pk, tile, xin, y, raw, hh, pad, act in layers:
+        pk.prepare(N, hh, hh, 1, pad, tile, stream=side.cuda_stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for _, pk, tile, xin, y, raw, hh, pad, act in layers:
+            pk.launch_act(xin.data_ptr(), y.data_ptr(), N, hh, hh, 1, pad, tile, act, stream=side.cuda_stream)
+    for rep in range(3):
+        x = rng.random((N, 8, H, H), dtype=np.float32) - 0.3
+        x0.copy_(torch.from_numpy(x))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [l[4].clone() for l in layers]
+        ref = x
+        for (w, pk, tile, xin, y, raw, hh, pad, act), g in zip(layers, got):  # eager, two passes, same buffers
+            pk.launch(xin.data_ptr(), raw.data_ptr(), N, hh, hh, 1, pad, tile)
+            T.relu_maxpool(raw.data_ptr(), y.data_ptr(), N, raw.shape[1], hh, hh, act)
+            torch.cuda.synchronize()
+            assert torch.equal(y, g), rep
+            ref = _np_relu_pool(oracle.host_conv2d(np.ascontiguousarray(ref), w, 1, pad), act)
+            assert max_rel_err(g.cpu().numpy(), ref) <= 1e-4, rep
+            ref = g.cpu().numpy()
+    for l in layers:
+        l[1].close()
