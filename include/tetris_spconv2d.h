@@ -285,6 +285,13 @@ int tetris_spconv2d_host(const float* h_input, const float* h_filter, float* h_o
 int tetris_spconv2d_spf_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
                              int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
                              void* stream, const char* layout, int apply_reorder, unsigned flags, float* ms_out);
+/* Replaces SparseConv2d_Baseline<float,int,int> (Tetris/baseline.cc:22-93), the first rung of the reference's
+ * ablation ladder: as tetris_spconv2d_spf_host, but the SparseFilter is built with apply_reorder = false (baseline.cc:44:
+ * the keep-as-is, CSR-like arrays of spconv2d_utils.h:38-61, no channel permutation) and those arrays feed the
+ * convolution (tetris_spconv2d_launch_spf_arrays with vec_width 0), run with the same fixed tile. */
+int tetris_spconv2d_baseline_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
+                                  int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
+                                  void* stream, const char* layout, float* ms_out);
 
 /* Times `repeat` back-to-back launches after `warm` untimed ones (TimingTetrisSparseConv2d,
  * Tetris/spconv2d.cc:29-69); mean milliseconds per launch in *ms_out. */

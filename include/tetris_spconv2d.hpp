@@ -6,6 +6,7 @@
 //   SparseConv2d<V,O,P,...>  Tetris/spconv2d_kernel.cuh:14-21 (launcher on the filter's device arrays)
 //   CudaSparseConv2d<V,O,P>  Tetris/spconv2d_kernel.cuh:7-12, Tetris/spconv2d.cc:332-367
 //   SparseConv2d_SPF<V,O,P>  Tetris/spf.cc:22-93
+//   SparseConv2d_Baseline<V,O,P>  Tetris/baseline.cc:22-93
 //   ReadConfigAndDataFromFile, PrintConv2dConfig, FloatEqual, TensorEqual   Tetris/tensor_utils.cc:17-82
 //
 // Only <float, int, int> exists, as in the reference (Tetris/spconv2d.cc:427, spconv2d_kernel.cu:197-200).
@@ -162,6 +163,25 @@ void SparseConv2d_SPF(float* h_input, float* h_filter, float* h_output, int batc
                                         layout.c_str(), apply_reorder, tetris_detail::build_flags(), &ms));
   std::cout << "Time of Ablation :" << ms << "ms"
             << "\n";
+}
+
+// Prints "Time of Baseline :<ms>ms" and "FLOPS of Baseline :<x>T" like Tetris/baseline.cc:82-83.
+template <typename ValueType, typename OffsetType, typename PositionType, typename Stream = void*>
+void SparseConv2d_Baseline(float* h_input, float* h_filter, float* h_output, int batch_size, int img_h, int img_w,
+                           int in_channel, int out_channel, int kernel_size, int stride, int padding, Stream stream,
+                           std::string layout, bool /*apply_reorder*/) {
+  float ms = 0.f;
+  TETRIS_CHECK(tetris_spconv2d_baseline_host(h_input, h_filter, h_output, batch_size, img_h, img_w, in_channel,
+                                             out_channel, kernel_size, stride, padding,
+                                             reinterpret_cast<void*>(stream), layout.c_str(), &ms));
+  const int out_h = (img_h + padding * 2 - kernel_size) / stride + 1;
+  const int out_w = (img_w + padding * 2 - kernel_size) / stride + 1;
+  std::cout << "Time of Baseline :" << ms << "ms"
+            << "\n";
+  std::cout << "FLOPS of Baseline :"
+            << (long long)out_h * out_w * batch_size * out_channel * in_channel * kernel_size * kernel_size * 2 * 1000 /
+                   (ms) / 1024 / 1024 / 1024 / 1024
+            << "T\n";
 }
 
 inline void PrintConv2dConfig(int64_t nnz, int batch_size, std::string /*layout*/, int img_h, int img_w, int in_channel,

@@ -21,7 +21,11 @@ def write_weight_file(path, w, H, W, pad, stride):
         f.write(" ".join(repr(float(v)) for v in w.reshape(-1)) + "\n")
 
 
-@pytest.mark.parametrize("exe", ["spconv2d_test", "spf_test"])
+ALL_CLIS = ["spconv2d_test", "para_test", "spf_test", "bank_sr_test", "filter_gr_test", "wo_bank_sr_test",
+            "wi_bank_sr_test", "baseline_test"]  # evalution/script/build_all.sh:14, build_ablation.sh:12-18
+
+
+@pytest.mark.parametrize("exe", ALL_CLIS)
 def test_cli_is_built_and_explains_itself(exe):
     p = subprocess.run([os.path.join(BIN, exe)], capture_output=True, text=True, timeout=60)
     assert p.returncode == 2 and "usage" in p.stderr
@@ -33,6 +37,12 @@ def test_cli_is_built_and_explains_itself(exe):
     ("spconv2d_test", (3, 24, 20, 20, 40, 3, 1, 1)),
     ("spconv2d_test", (2, 16, 15, 15, 33, 1, 2, 0)),
     ("spf_test", (2, 24, 20, 20, 40, 3, 1, 1)),
+    ("bank_sr_test", (2, 24, 20, 20, 40, 3, 1, 1)),
+    ("filter_gr_test", (2, 24, 20, 20, 40, 3, 1, 1)),
+    ("wo_bank_sr_test", (3, 20, 14, 14, 70, 3, 2, 1)),
+    ("baseline_test", (2, 24, 20, 20, 40, 3, 1, 1)),
+    ("baseline_test", (1, 40, 9, 9, 33, 1, 1, 0)),
+    ("para_test", (2, 24, 20, 20, 40, 3, 1, 1)),
 ])
 def test_cli_output_and_tensors(oracle, tmp_path, exe, shape):
     N, C, H, W, K, ks, stride, pad = shape
@@ -49,9 +59,10 @@ def test_cli_output_and_tensors(oracle, tmp_path, exe, shape):
                   r"in_channel = (\d+), out_channel = (\d+), kernel_size = (\d+), padding = (\d+), stride = (\d+)", out)
     assert m and [int(v) for v in m.groups()[1:]] == [nnz, N, H, W, C, K, ks, pad, stride]
     assert abs(float(m.group(1)) - (1.0 - nnz / w.size)) < 1e-5
-    if exe == "spconv2d_test":  # the lines evalution/conv2d_timing.py:51-79 parses
-        t = re.search(r"Time of Spconv2d :([0-9.e-]+)ms", out)
-        fl = re.search(r"FLOPS of Spconv2d :([0-9.e+-]+)T", out)
+    if exe in ("spconv2d_test", "para_test", "baseline_test"):  # the lines evalution/conv2d_timing.py:51-79 parses
+        who = "Baseline" if exe == "baseline_test" else "Spconv2d"  # Tetris/baseline.cc:82-83, spconv2d.cc:357-358
+        t = re.search(r"Time of %s :([0-9.e-]+)ms" % who, out)
+        fl = re.search(r"FLOPS of %s :([0-9.e+-]+)T" % who, out)
         assert t and fl and float(t.group(1)) > 0
         oh, ow = (H + 2 * pad - ks) // stride + 1, (W + 2 * pad - ks) // stride + 1
         want = oh * ow * N * K * C * ks * ks * 2 * 1000 / float(t.group(1)) / 1024 ** 4
@@ -126,6 +137,55 @@ def test_timing_driver_parses_and_writes_the_reference_csv(tmp_path):
     bad.chmod(0o755)
     with pytest.raises(RuntimeError):
         timing.time_layer(str(bad), str(folder / "conv_0"), 1)
+
+
+def test_ablation_driver_writes_the_reference_csv(tmp_path):
+    # host logic of the ladder loop (counterpart of evalution/ablation_timing.py), with stand-in binaries
+    from tetris_amd import timing
+
+    folder = tmp_path / "vgg19-90-acc"
+    folder.mkdir()
+    rng = np.random.default_rng(1)
+    for i in range(2):
+        timing.write_weight_file(str(folder / ("conv_%d" % i)), sparse_filter(rng, 8, 4, 3, 0.5), 9, 9, 1, 1)
+    bins = tmp_path / "bin"
+    bins.mkdir()
+    lines = {"baseline_test": "Time of Baseline :0.5ms\nFLOPS of Baseline :1.5T\n", "spf_test": "Time of Ablation :0.4ms\n",
+             "bank_sr_test": "Time of Ablation :0.3ms\n", "filter_gr_test": "Time of Ablation :0.25ms\n",
+             "para_test": "Time of Spconv2d :0.125ms\nFLOPS of Spconv2d :6T\n"}
+    for name, text in lines.items():
+        f = bins / name
+        f.write_text("#!/bin/sh\ncat <<'EOT'\n[Config] sparsity = 0.5, nnz = 144, batch_size = 4, kernel_size = 3\n" + text + "EOT\n")
+        f.chmod(0o755)
+    csv, rows = timing.ablation_folder(str(bins), str(folder), 4, str(tmp_path / "logs"))
+    assert os.path.basename(csv) == "ablation_a.csv"
+    assert open(csv).read().splitlines() == [",op_name,Baseline,SPF,Bank-SR,Filter-GR,Para",
+                                             "0,conv_0,0.50000,0.40000,0.30000,0.25000,0.12500",
+                                             "1,conv_1,0.50000,0.40000,0.30000,0.25000,0.12500"]
+    log = open(str(tmp_path / "logs" / "ablation_a.log")).read()
+    assert log.count("# Run[") == 2 and "Bank-SR: time = 0.30000ms" in log and "'kernel_size': '3'" in log
+    (bins / "para_test").unlink()
+    with pytest.raises(SystemExit):
+        timing.main(["--ablation", "--weights", str(folder), "--bin-dir", str(bins), "--log-dir", str(tmp_path / "l2")])
+
+
+@pytest.mark.gpu
+def test_ablation_driver_on_the_real_binaries(tmp_path):
+    from tetris_amd import timing
+
+    folder = tmp_path / "net-80"
+    folder.mkdir()
+    rng = np.random.default_rng(2)
+    timing.write_weight_file(str(folder / "a_3x3"), sparse_filter(rng, 64, 32, 3, 0.8), 28, 28, 1, 1)
+    timing.write_weight_file(str(folder / "b_1x1"), sparse_filter(rng, 48, 64, 1, 0.8), 14, 14, 0, 1)
+    csv, rows = timing.ablation_folder(BIN, str(folder), 4, str(tmp_path / "logs"))
+    assert [op for op, _ in rows] == ["a_3x3", "b_1x1"]
+    assert all(len(t) == 5 and all(0 < v < 50 for v in t) for _, t in rows)
+    # every rung computes the convolution: the reference's own check, through each binary
+    for exe in [b for b, _ in timing.LADDER]:
+        p = subprocess.run([os.path.join(BIN, exe), str(folder / "a_3x3"), "2", "--check"], capture_output=True, text=True,
+                           timeout=120)
+        assert p.returncode == 0 and "Sparse Pass." in p.stdout, (exe, p.stdout[-500:], p.stderr[-500:])
 
 
 @pytest.mark.gpu

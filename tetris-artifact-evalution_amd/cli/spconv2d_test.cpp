@@ -1,12 +1,24 @@
-// spconv2d_test <weight_file> [batch] [--seed S] [--dump FILE] [--check]      (built twice: spconv2d_test and, with
-// -DTETRIS_CLI_SPF, spf_test)
+// spconv2d_test <weight_file> [batch] [--seed S] [--dump FILE] [--check]
 //
-// Counterpart of the reference's per-layer binaries: main of Tetris/spconv2d.cc:369-450 (spconv2d_test.o,
-// "Time of Spconv2d :<ms>ms" / "FLOPS of Spconv2d :<x>T") and of Tetris/spf.cc:95-176 (spf_test.o,
-// "Time of Ablation :<ms>ms").  It reads one pruned layer in the reference's text format, makes a random
-// input, runs the host-to-host entry point (upload, pack, tile selection, 30 warm-up + 100 timed
-// launches, download) and prints the same lines, so a loop over weight files that parses the reference's
-// stdout (evalution/conv2d_timing.py:51-79) can drive it unchanged.
+// One source, built once per binary of the reference (its names without the ".o"):
+//   spconv2d_test, para_test   Tetris/spconv2d.cc:369-450 with -DBANK_OPTIMIZE -DREORDER_OUT_CHANNEL
+//                              (evalution/script/build_all.sh:14, build_ablation.sh:16): the library's path, tile
+//                              from its table; prints "Time of Spconv2d :<ms>ms" / "FLOPS of Spconv2d :<x>T"
+//   spf_test, bank_sr_test, filter_gr_test, wo_bank_sr_test, wi_bank_sr_test   (-DTETRIS_CLI_SPF)
+//                              Tetris/spf.cc:95-176 with no switch, -DBANK_OPTIMIZE, both, -DREORDER_OUT_CHANNEL
+//                              alone, both (build_ablation.sh:13-18): the fixed configuration on the SparseFilter's
+//                              device arrays; prints "Time of Ablation :<ms>ms"
+//   baseline_test              (-DTETRIS_CLI_BASELINE) Tetris/baseline.cc:95-176: the same on the keep-as-is,
+//                              CSR-like arrays; prints "Time of Baseline :<ms>ms" / "FLOPS of Baseline :<x>T"
+// BANK_OPTIMIZE makes the SparseFilter run Bank-SR, as in the reference.  That pass orders entries for the banks of
+// the reference's kernel; what keeps this library's kernel free of LDS bank conflicts is the pitch rule of its LDS
+// tiles, so the binaries of the fixed configuration built WITHOUT BANK_OPTIMIZE also switch that rule off
+// (TETRIS_OPT_NO_BANK_RULE): the rung "Bank-SR" of the ladder then measures conflict avoidance here as it does there.
+//
+// Each reads one pruned layer in the reference's text format, makes a random input, runs the host-to-host entry
+// point (upload, pack, 30 warm-up + 100 timed launches, download) and prints the reference's lines, so a loop over
+// weight files that parses the reference's stdout (evalution/conv2d_timing.py:51-79, ablation_timing.py:15-57) can
+// drive it unchanged.
 //
 // The reference seeds rand() with time(0) (Tetris/spconv2d.cc:377); here the input comes from a
 // seeded generator so that a run can be repeated, and --dump writes input and output tensors (raw
@@ -24,9 +36,7 @@
 #include <iostream>
 #include <string>
 
-#define BANK_OPTIMIZE        // the production variant: evalution/script/build_all.sh:14
-#define REORDER_OUT_CHANNEL
-#include "tetris_spconv2d.hpp"
+#include "tetris_spconv2d.hpp"  // BANK_OPTIMIZE / REORDER_OUT_CHANNEL come from the build line, as in the reference
 
 namespace {
 
@@ -118,7 +128,16 @@ int main(int argc, char* argv[]) {
 
   hipStream_t stream;
   CLI_HIP(hipStreamCreate(&stream));
-#ifdef TETRIS_CLI_SPF
+#if (defined(TETRIS_CLI_SPF) || defined(TETRIS_CLI_BASELINE)) && !defined(BANK_OPTIMIZE)
+  if (tetris_options_set(tetris_options_get() | TETRIS_OPT_NO_BANK_RULE) != TETRIS_OK) {
+    std::fprintf(stderr, "%s\n", tetris_last_error());
+    return 1;
+  }
+#endif
+#if defined(TETRIS_CLI_BASELINE)
+  SparseConv2d_Baseline<float, int, int>(h_input, h_filter, h_sparse, batch_size, img_h, img_w, in_channel, out_channel,
+                                         kernel_size, stride, padding, stream, layout, false);
+#elif defined(TETRIS_CLI_SPF)
   SparseConv2d_SPF<float, int, int>(h_input, h_filter, h_sparse, batch_size, img_h, img_w, in_channel, out_channel,
                                     kernel_size, stride, padding, stream, layout, apply_reorder);
 #else

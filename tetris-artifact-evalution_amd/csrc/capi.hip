@@ -357,9 +357,12 @@ tetris_tile fixed_spf_tile(int N, int H, int W, int C, int K, int ks, int stride
 // Shared body of the two host-to-host entry points.  spf_path: the reference's SparseConv2d_SPF (Tetris/spf.cc:22-93):
 // SparseFilter with TILE_IC = 128 and apply_reorder = true whatever the caller passed (:43-44), its device arrays handed
 // to the launcher, one fixed tile.
+// baseline: the reference's SparseConv2d_Baseline (Tetris/baseline.cc:22-93): SparseFilter with TILE_IC = 128 and
+// apply_reorder = false (the keep-as-is, CSR-like arrays of spconv2d_utils.h:38-61) handed to the launcher, the same
+// fixed tile.
 int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K, int ks,
               int stride, int pad, hipStream_t stream, bool apply_reorder, bool spf_path, unsigned spf_flags,
-              float* ms_out) {
+              float* ms_out, bool baseline = false) {
   if (!h_in || !h_filter || !h_out) return fail(TETRIS_EINVAL, "null argument");
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || stride <= 0 || pad < 0)
     return fail(TETRIS_EINVAL, "bad conv shape");
@@ -380,14 +383,14 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
   int rc;
   tetris_g950* run = nullptr;
   if (spf_path) {
-    rc = tetris_spf_create(h_filter, C, K, ks, 128, 1, 1, spf_flags, &spf);
+    rc = tetris_spf_create(h_filter, C, K, ks, 128, baseline ? 0 : 1, 1, spf_flags, &spf);
     if (rc) return done(rc);
     tetris_spf_arrays a{};
     rc = tetris_spf_device_arrays(spf, &a);
     if (rc) return done(rc);
     const tetris_tile fixed = fixed_spf_tile(N, H, W, C, K, ks, stride, pad);
-    rc = view_pack(a.offsets, a.oc_permutation, a.position, a.values, N, H, W, C, K, ks, stride, pad, 128, 4, &fixed, stream,
-                   &run, &tile);
+    rc = view_pack(a.offsets, baseline ? nullptr : a.oc_permutation, a.position, a.values, N, H, W, C, K, ks, stride, pad,
+                   128, baseline ? 0 : 4, &fixed, stream, &run, &tile);
     if (rc) return done(rc);
   } else {
     rc = choose_tile(N, H, W, C, K, ks, stride, pad, &tile);
@@ -755,6 +758,13 @@ int tetris_spconv2d_spf_host(const float* h_in, const float* h_filter, float* h_
   if (flags & ~(TETRIS_BANK_OPTIMIZE | TETRIS_REORDER_OUT_CHANNEL)) return fail(TETRIS_EINVAL, "unknown flags 0x%x", flags);
   return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream), true, true,
                    flags, ms_out);
+}
+
+int tetris_spconv2d_baseline_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C,
+                                  int K, int ks, int stride, int pad, void* stream, const char* layout, float* ms_out) {
+  (void)layout;
+  return conv_host(h_in, h_filter, h_out, N, H, W, C, K, ks, stride, pad, static_cast<hipStream_t>(stream), false, true,
+                   0u, ms_out, true);
 }
 
 int tetris_read_weight_file(const char* path, int32_t header[8], float** h_filter_out, int64_t* nnz_out) {

@@ -2,6 +2,7 @@
 (its Tetris column) on this library's command-line driver.
 
     python -m tetris_amd.timing --weights DIR [--batch 1 4 8 16] [--log-dir DIR] [--bin PATH]
+    python -m tetris_amd.timing --ablation --weights DIR [--batch 4] [--log-dir DIR] [--bin-dir DIR]
     python -m tetris_amd.timing --write-suite vgg19 DIR        # the synthetic suite as weight files
     python -m tetris_amd.timing --write-masks MASKS.npz DIR    # a pruned network's layers (seeded values)
 
@@ -12,6 +13,12 @@ process and reads the lines the reference's harness reads (conv2d_timing.py:51-7
 (conv2d_timing.py:101-198), `<folder>_batch_<N>.csv` (columns: row index, op_name, spconv2d in ms with five decimals)
 and `<folder>_batch_<N>.log`.  Only the Tetris column exists here: the vendor baselines of the reference are not part
 of this library.
+
+--ablation is the counterpart of evalution/ablation_timing.py: every layer goes through the five binaries of the
+reference's ladder (ablation_timing.py:109-115: baseline_test, spf_test, bank_sr_test, filter_gr_test, para_test, built
+by this package's Makefile with the switches of evalution/script/build_ablation.sh:12-16) and the times land in
+`ablation_a.csv` (columns: row index, op_name, Baseline, SPF, Bank-SR, Filter-GR, Para) and `ablation_a.log`, as there
+(:79-80, :143-144).
 """
 import argparse
 import os
@@ -68,6 +75,39 @@ def time_folder(binary, folder, batch, log_dir):
     return csv, rows
 
 
+LADDER = [("baseline_test", "Baseline"), ("spf_test", "SPF"), ("bank_sr_test", "Bank-SR"),
+          ("filter_gr_test", "Filter-GR"), ("para_test", "Para")]  # evalution/ablation_timing.py:109-115
+
+
+def ablation_folder(bin_dir, folder, batch, log_dir):
+    """One row per weight file, one column per rung of the ladder; -> (csv path, rows of (op, [ms per rung]))."""
+    folder = folder.rstrip("/")
+    os.makedirs(log_dir, exist_ok=True)
+    rows = []
+    with open(os.path.join(log_dir, "ablation_a.log"), "w") as log:
+        for idx, op in enumerate(sorted(os.listdir(folder))):
+            path = os.path.join(folder, op)
+            if not os.path.isfile(path):
+                continue
+            log.write("# Run[%d]: %s\n" % (idx, path))
+            times = []
+            for k, (binary, name) in enumerate(LADDER):
+                config, ms, tflops = time_layer(os.path.join(bin_dir, binary), path, batch)
+                if k == 0:
+                    log.write("%r\n" % (config,))
+                log.write("%s: time = %.5fms\n" % (name, ms))
+                times.append(ms)
+            log.write("-" * 84 + "\n\n")
+            log.flush()
+            rows.append((op, times))
+    csv = os.path.join(log_dir, "ablation_a.csv")
+    with open(csv, "w") as f:
+        f.write(",op_name,%s\n" % ",".join(name for _, name in LADDER))
+        for i, (op, times) in enumerate(rows):
+            f.write("%d,%s,%s\n" % (i, op, ",".join("%.5f" % t for t in times)))
+    return csv, rows
+
+
 def write_weight_file(path, w, H, W, pad, stride, groups=1):
     K, C, ks, _ = w.shape
     with open(path, "w") as f:
@@ -93,6 +133,8 @@ def main(argv=None):
     ap.add_argument("--batch", nargs="+", type=int, default=[1])
     ap.add_argument("--log-dir", default="timing_out")
     ap.add_argument("--bin", default=os.path.join(here, "bin", "spconv2d_test"))
+    ap.add_argument("--ablation", action="store_true", help="time the five binaries of the ablation ladder instead")
+    ap.add_argument("--bin-dir", default=os.path.join(here, "bin"), help="where the ladder's binaries are (--ablation)")
     ap.add_argument("--write-suite", nargs=2, metavar=("SUITE", "DIR"))
     ap.add_argument("--write-masks", nargs=2, metavar=("NPZ", "DIR"))
     args = ap.parse_args(argv)
@@ -101,7 +143,17 @@ def main(argv=None):
         layers = W.SUITES[args.write_suite[0]]() if args.write_suite else W.pruned_suite(args.write_masks[0])
         out_dir = (args.write_suite or args.write_masks)[1]
         print("wrote %d weight files to %s" % (write_layers(layers, out_dir), out_dir))
-    if args.weights:
+    if args.weights and args.ablation:
+        missing = [b for b, _ in LADDER if not os.path.isfile(os.path.join(args.bin_dir, b))]
+        if missing:
+            sys.exit("timing: %s not built in %s (make -C %s)" % (", ".join(missing), args.bin_dir, here))
+        for n in args.batch:
+            log_dir = args.log_dir if len(args.batch) == 1 else os.path.join(args.log_dir, "batch_%d" % n)
+            csv, rows = ablation_folder(args.bin_dir, args.weights, n, log_dir)
+            sums = [sum(t[k] for _, t in rows) for k in range(len(LADDER))]
+            print("batch %d: %d layers; %s -> %s" % (n, len(rows), ", ".join("%s %.3f ms" % (name, v) for (_, name), v in
+                                                                          zip(LADDER, sums)), csv), flush=True)
+    elif args.weights:
         if not os.path.isfile(args.bin):
             sys.exit("timing: %s is not built (make -C %s)" % (args.bin, here))
         for n in args.batch:
