@@ -152,7 +152,7 @@ void CudaSparseConv2d(float* h_input, float* h_filter, float* h_output, int batc
             << "T\n";
 }
 
-// Prints "Time of Ablation :<ms>ms" like Tetris/spf.cc:83.
+// Prints "Time of Ablation :<ms>ms" and "FLOPS of Ablation :<x>T" like Tetris/spf.cc:83-84.
 template <typename ValueType, typename OffsetType, typename PositionType, typename Stream = void*>
 void SparseConv2d_SPF(float* h_input, float* h_filter, float* h_output, int batch_size, int img_h, int img_w,
                       int in_channel, int out_channel, int kernel_size, int stride, int padding, Stream stream,
@@ -161,8 +161,14 @@ void SparseConv2d_SPF(float* h_input, float* h_filter, float* h_output, int batc
   TETRIS_CHECK(tetris_spconv2d_spf_host(h_input, h_filter, h_output, batch_size, img_h, img_w, in_channel,
                                         out_channel, kernel_size, stride, padding, reinterpret_cast<void*>(stream),
                                         layout.c_str(), apply_reorder, tetris_detail::build_flags(), &ms));
+  const int out_h = (img_h + padding * 2 - kernel_size) / stride + 1;
+  const int out_w = (img_w + padding * 2 - kernel_size) / stride + 1;
   std::cout << "Time of Ablation :" << ms << "ms"
             << "\n";
+  std::cout << "FLOPS of Ablation :"
+            << (long long)out_h * out_w * batch_size * out_channel * in_channel * kernel_size * kernel_size * 2 * 1000 /
+                   (ms) / 1024 / 1024 / 1024 / 1024
+            << "T\n";
 }
 
 // Prints "Time of Baseline :<ms>ms" and "FLOPS of Baseline :<x>T" like Tetris/baseline.cc:82-83.

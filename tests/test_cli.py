@@ -253,3 +253,49 @@ def test_memory_metric_on_the_real_binaries(tmp_path):
         assert r[v]["dispatches"] == 130 and r[v]["SQ_INSTS_LDS"] > 0 and r[v]["SQ_LDS_IDX_ACTIVE"] > 0  # 30 warm + 100 timed
     assert r["wi"]["SQ_LDS_BANK_CONFLICT"] <= 0.01 * r["wi"]["SQ_LDS_IDX_ACTIVE"]
     assert r["wo"]["SQ_LDS_BANK_CONFLICT"] >= r["wi"]["SQ_LDS_BANK_CONFLICT"]
+
+
+def test_timing_driver_vendor_columns(tmp_path, monkeypatch):
+    # --vendors: the reference's cudnn / cusparse columns of conv2d_timing.py, here miopen / rocsparse, before the
+    # library's own column; the children are stand-ins
+    from tetris_amd import timing
+
+    folder = tmp_path / "net-90"
+    folder.mkdir()
+    rng = np.random.default_rng(3)
+    timing.write_weight_file(str(folder / "conv_0"), sparse_filter(rng, 8, 4, 3, 0.5), 9, 9, 1, 1)
+    fake = tmp_path / "fake_bin"
+    fake.write_text("#!/bin/sh\ncat <<'EOT'\n" + CANNED + "EOT\n")
+    fake.chmod(0o755)
+    monkeypatch.setattr(timing, "time_vendor", lambda kind, path, batch: ({}, 0.5 if kind == "dense" else 7.25, 1.0))
+    csv, rows = timing.time_folder(str(fake), str(folder), 4, str(tmp_path / "logs"), vendors=True)
+    assert open(csv).read().splitlines() == [",op_name,miopen,rocsparse,spconv2d", "0,conv_0,0.50000,7.25000,%.5f" % 0.012345]
+    log = open(str(tmp_path / "logs" / "net-90_batch_4.log")).read()
+    assert "miopen: time = 0.50000ms" in log and "rocsparse: time = 7.25000ms" in log and "spconv2d: time = 0.0123" in log
+
+
+def test_vendor_driver_explains_itself(capsys):
+    from tetris_amd import vendor_test
+
+    assert vendor_test.main(["dense"]) == 2
+    assert capsys.readouterr().out.startswith("args : 2 vendor_test dense")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,label", [("dense", "MIOpen"), ("csr", "Rocsparse")])
+def test_vendor_driver_on_the_gpu(tmp_path, kind, label):
+    # one child process per layer and vendor, the reference's stdout lines, the result checked against a dense conv
+    import sys
+    from tetris_amd import timing
+
+    rng = np.random.default_rng(6)
+    wf = str(tmp_path / "layer")
+    timing.write_weight_file(wf, sparse_filter(rng, 24, 16, 3, 0.8), 14, 14, 1, 1)
+    env = dict(os.environ, PYTHONPATH=os.path.join(ROOT, "tetris-artifact-evalution_amd"))
+    p = subprocess.run([sys.executable, "-m", "tetris_amd.vendor_test", kind, wf, "2", "--check"], capture_output=True,
+                       text=True, timeout=300, env=env)
+    assert p.returncode == 0, p.stdout[-800:] + p.stderr[-800:]
+    cfg, ms, tf = timing.parse_output(p.stdout)
+    assert cfg["out_channel"] == "24" and cfg["batch_size"] == "2" and ms > 0 and tf > 0
+    assert "Time of %s :" % label in p.stdout and "Sparse Pass." in p.stdout
+    assert timing.time_vendor(kind, wf, 2)[1] > 0

@@ -1,7 +1,7 @@
 """Per-layer timing over a folder of weight files: the counterpart of the reference's evalution/conv2d_timing.py
 (its Tetris column) on this library's command-line driver.
 
-    python -m tetris_amd.timing --weights DIR [--batch 1 4 8 16] [--log-dir DIR] [--bin PATH]
+    python -m tetris_amd.timing --weights DIR [--batch 1 4 8 16] [--log-dir DIR] [--bin PATH] [--vendors]
     python -m tetris_amd.timing --ablation --weights DIR [--batch 4] [--log-dir DIR] [--bin-dir DIR]
     python -m tetris_amd.timing --write-suite vgg19 DIR        # the synthetic suite as weight files
     python -m tetris_amd.timing --write-masks MASKS.npz DIR    # a pruned network's layers (seeded values)
@@ -11,8 +11,9 @@ OIHW values, Tetris/tensor_utils.cc:55-82) and batch size it starts `bin/spconv2
 process and reads the lines the reference's harness reads (conv2d_timing.py:51-79): `[Config] k = v, ...`,
 `Time of Spconv2d :<ms>ms`, `FLOPS of Spconv2d :<x>T`.  Per batch size it writes, like the reference
 (conv2d_timing.py:101-198), `<folder>_batch_<N>.csv` (columns: row index, op_name, spconv2d in ms with five decimals)
-and `<folder>_batch_<N>.log`.  Only the Tetris column exists here: the vendor baselines of the reference are not part
-of this library.
+and `<folder>_batch_<N>.log`.  --vendors adds the columns `miopen` and `rocsparse` before it, the counterparts on this
+machine of the reference's `cudnn` and `cusparse` columns (tetris_amd.vendor_test, one child process per layer and
+column like the reference's cudnn_test.o / cusparse_test.o); the Sputnik columns have no counterpart here.
 
 --ablation is the counterpart of evalution/ablation_timing.py: every layer goes through the five binaries of the
 reference's ladder (ablation_timing.py:109-115: baseline_test, spf_test, bank_sr_test, filter_gr_test, para_test, built
@@ -52,7 +53,21 @@ def time_layer(binary, weight_file, batch, timeout=600):
     return parse_output(p.stdout)
 
 
-def time_folder(binary, folder, batch, log_dir):
+VENDORS = [("dense", "miopen"), ("csr", "rocsparse")]  # the reference's cudnn and cusparse columns (conv2d_timing.py:24-28)
+
+
+def time_vendor(kind, weight_file, batch, timeout=1200):
+    """One vendor baseline of one layer, in a child process like every other column (tetris_amd.vendor_test)."""
+    here = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, PYTHONPATH=here + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    cmd = [sys.executable, "-m", "tetris_amd.vendor_test", kind, weight_file, str(batch)]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout, env=env)
+    if p.returncode != 0:
+        raise RuntimeError("%s: exit %d\n%s%s" % (" ".join(cmd), p.returncode, p.stdout[-2000:], p.stderr[-2000:]))
+    return parse_output(p.stdout)
+
+
+def time_folder(binary, folder, batch, log_dir, vendors=False):
     folder = folder.rstrip("/")
     tag = "%s_batch_%d" % (os.path.basename(folder), batch)
     os.makedirs(log_dir, exist_ok=True)
@@ -63,15 +78,19 @@ def time_folder(binary, folder, batch, log_dir):
             if not os.path.isfile(path):
                 continue
             log.write("# Run[%d]: %s\n" % (idx, path))
+            others = [(name,) + time_vendor(kind, path, batch)[1:] for kind, name in VENDORS] if vendors else []
             config, ms, tflops = time_layer(binary, path, batch)
-            log.write("%r\n%s: time = %.5fms, FLOPS = %.5fT\n%s\n\n" % (config, VENDOR, ms, tflops, "-" * 84))
+            log.write("%r\n" % (config,))
+            for name, vms, vtf in others:
+                log.write("%s: time = %.5fms, FLOPS = %.5fT\n" % (name, vms, vtf))
+            log.write("%s: time = %.5fms, FLOPS = %.5fT\n%s\n\n" % (VENDOR, ms, tflops, "-" * 84))
             log.flush()
-            rows.append((op, ms))
+            rows.append((op, ms) if not vendors else (op, ms, [v[1] for v in others]))
     csv = os.path.join(log_dir, tag + ".csv")
     with open(csv, "w") as f:
-        f.write(",op_name,%s\n" % VENDOR)
-        for i, (op, ms) in enumerate(rows):
-            f.write("%d,%s,%.5f\n" % (i, op, ms))
+        f.write(",op_name,%s%s\n" % ("".join(name + "," for _, name in VENDORS) if vendors else "", VENDOR))
+        for i, row in enumerate(rows):
+            f.write("%d,%s,%s%.5f\n" % (i, row[0], "".join("%.5f," % v for v in row[2]) if vendors else "", row[1]))
     return csv, rows
 
 
@@ -133,6 +152,8 @@ def main(argv=None):
     ap.add_argument("--batch", nargs="+", type=int, default=[1])
     ap.add_argument("--log-dir", default="timing_out")
     ap.add_argument("--bin", default=os.path.join(here, "bin", "spconv2d_test"))
+    ap.add_argument("--vendors", action="store_true", help="also time the vendor's dense convolution and CSR product per "
+                    "layer (columns miopen, rocsparse: the reference's cudnn and cusparse columns)")
     ap.add_argument("--ablation", action="store_true", help="time the five binaries of the ablation ladder instead")
     ap.add_argument("--bin-dir", default=os.path.join(here, "bin"), help="where the ladder's binaries are (--ablation)")
     ap.add_argument("--write-suite", nargs=2, metavar=("SUITE", "DIR"))
@@ -157,8 +178,8 @@ def main(argv=None):
         if not os.path.isfile(args.bin):
             sys.exit("timing: %s is not built (make -C %s)" % (args.bin, here))
         for n in args.batch:
-            csv, rows = time_folder(args.bin, args.weights, n, args.log_dir)
-            print("batch %d: %d layers, %.3f ms in total -> %s" % (n, len(rows), sum(ms for _, ms in rows), csv), flush=True)
+            csv, rows = time_folder(args.bin, args.weights, n, args.log_dir, vendors=args.vendors)
+            print("batch %d: %d layers, %.3f ms in total -> %s" % (n, len(rows), sum(r[1] for r in rows), csv), flush=True)
     elif not (args.write_suite or args.write_masks):
         ap.error("nothing to do: give --weights, --write-suite or --write-masks")
 
