@@ -272,6 +272,8 @@ def test_timing_driver_vendor_columns(tmp_path, monkeypatch):
     assert open(csv).read().splitlines() == [",op_name,miopen,rocsparse,spconv2d", "0,conv_0,0.50000,7.25000,%.5f" % 0.012345]
     log = open(str(tmp_path / "logs" / "net-90_batch_4.log")).read()
     assert "miopen: time = 0.50000ms" in log and "rocsparse: time = 7.25000ms" in log and "spconv2d: time = 0.0123" in log
+    sp = dict(timing.geo_mean_speedups(rows + [("conv_1", 0.25, [1.0, 1.0])]))  # evalution/overall_speedup.py:45-51
+    assert abs(sp["miopen"] - (0.5 / 0.012345 * 4.0) ** 0.5) < 1e-9 and abs(sp["rocsparse"] - (7.25 / 0.012345 * 4.0) ** 0.5) < 1e-9
 
 
 def test_vendor_driver_explains_itself(capsys):

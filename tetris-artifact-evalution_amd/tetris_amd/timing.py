@@ -67,6 +67,17 @@ def time_vendor(kind, weight_file, batch, timeout=1200):
     return parse_output(p.stdout)
 
 
+def geo_mean_speedups(rows):
+    """Geometric mean over the layers of vendor time / library time, per vendor column, as the reference's summary
+    prints it (evalution/overall_speedup.py:45-51); rows as time_folder returns them with vendors=True."""
+    import math
+    out = []
+    for k, (_, name) in enumerate(VENDORS):
+        ratios = [r[2][k] / r[1] for r in rows if r[1] > 0 and r[2][k] > 0]
+        out.append((name, math.exp(sum(math.log(v) for v in ratios) / len(ratios)) if ratios else float("nan")))
+    return out
+
+
 def time_folder(binary, folder, batch, log_dir, vendors=False):
     folder = folder.rstrip("/")
     tag = "%s_batch_%d" % (os.path.basename(folder), batch)
@@ -180,6 +191,9 @@ def main(argv=None):
         for n in args.batch:
             csv, rows = time_folder(args.bin, args.weights, n, args.log_dir, vendors=args.vendors)
             print("batch %d: %d layers, %.3f ms in total -> %s" % (n, len(rows), sum(r[1] for r in rows), csv), flush=True)
+            if args.vendors:
+                for name, sp in geo_mean_speedups(rows):
+                    print("# Compare to %s : Geo Mean Speedup = %.2fx" % (name, sp), flush=True)
     elif not (args.write_suite or args.write_masks):
         ap.error("nothing to do: give --weights, --write-suite or --write-masks")
 
