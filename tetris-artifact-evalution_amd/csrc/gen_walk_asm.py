@@ -114,23 +114,34 @@ def walk(nq, variant="", share=1):
     # that rotate with every batch.  Left alone the SIMD serves its oldest wave first: that wave finishes its stage
     # early and idles at the barrier while the youngest runs the tail of the stage alone, too slowly to fill the
     # SIMD by itself.
+    # A stream is padded to whole batches with entries of weight zero.  With single-entry records the last batch of a
+    # call gets a copy of the body of its own (label 5) that leaves at the first zero weight (label 8): pads cost no
+    # FMAs.  (Real entries never carry +0.0: only non-zeros are packed.  In a stream of pairs a zero weight also marks
+    # the missing half of a pair, so those loops run every entry.)
+    last_exits = share == 1
+    if last_exits:
+        L.append("s_cmp_eq_u32 %[nb], 1")
+        L.append("s_cbranch_scc1 5f")
     for k in (1, 2, 3):
         L.append("s_cmp_eq_u32 %%[ph], %d" % k)
         L.append("s_cbranch_scc1 %df" % (k + 1))
-    for k in range(4):
-        L.append("%d:" % (k + 1))
-        L.append("s_setprio %d" % k)
+
+    def body(prio, exits):
+        L.append("s_setprio %d" % prio)
         L.append("s_load_dwordx16 s[52:67], s[72:73], 0x0")  # the batch after this one (may belong to the next stream)
         L.append("s_add_u32 s72, s72, 64")
         L.append("s_addc_u32 s73, s73, 0")
         refill_at = R - ahead  # first record whose look-ahead record lies in the next batch
         for r in range(R):
+            if exits and r > 0:  # (a call is never made for an empty stream: the first entry of a batch is real)
+                L.append("s_cmp_eq_u32 s%d, 0" % (37 + 2 * r))
+                L.append("s_cbranch_scc1 8f")
             if r == refill_at:
                 # the next batch must have arrived; its addresses replace the ones all consumed by now
                 L.append("s_waitcnt lgkmcnt(0)")
-                L += addresses(c, 52)
+                L.extend(addresses(c, 52))
             la = r + ahead  # record whose reads are issued now
-            L += reads(c, la % nbuf, c["a0"] + (la % R))
+            L.extend(reads(c, la % nbuf, c["a0"] + (la % R)))
             for kk in range(share):
                 e = r * share + kk
                 L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
@@ -138,15 +149,34 @@ def walk(nq, variant="", share=1):
                     L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
                 else:
                     L.append("s_nop 0")  # keeps one instruction between the write of M0 and the indexed VALU use
-                L += fmas(c, r % nbuf, 37 + 2 * e)
+                L.extend(fmas(c, r % nbuf, 37 + 2 * e))
+
+    def advance():
         for i in range(8):
             L.append("s_mov_b64 s[%d:%d], s[%d:%d]" % (36 + 2 * i, 37 + 2 * i, 52 + 2 * i, 53 + 2 * i))
+
+    for k in range(4):
+        L.append("%d:" % (k + 1))
+        body(k, False)
+        advance()
         L.append("s_sub_u32 %[nb], %[nb], 1")
-        L.append("s_cmp_lg_u32 %[nb], 0")
-        if k < 3:
-            L.append("s_cbranch_scc0 9f")
+        if last_exits:
+            L.append("s_cmp_eq_u32 %[nb], 1")
+            L.append("s_cbranch_scc1 5f")
+            if k == 3:
+                L.append("s_branch 1b")
         else:
-            L.append("s_cbranch_scc1 1b")
+            L.append("s_cmp_lg_u32 %[nb], 0")
+            if k < 3:
+                L.append("s_cbranch_scc0 9f")
+            else:
+                L.append("s_cbranch_scc1 1b")
+    if last_exits:
+        L.append("5:")
+        body(1, True)
+        L.append("8:")
+        L.append("s_waitcnt lgkmcnt(0)")  # the next batch has arrived (an early exit may come before the refill's wait)
+        advance()
     L.append("9:")
     L.append("s_setprio 3")  # what follows a walk (issuing the staging loads, reaching the barrier) should not wait
     L.append("s_waitcnt lgkmcnt(0)")  # drain the look-ahead reads (their data is not used)
