@@ -98,10 +98,8 @@ def walk(nq, variant="", share=1):
     nbuf = min(c["nbuf"], R)
     ahead = nbuf - 1                     # records of look-ahead
     L = []
-    for i in range(8):
-        L.append("s_mov_b64 s[%d:%d], %%[c%d]" % (36 + 2 * i, 37 + 2 * i, i))
-    L.append("s_mov_b32 s72, %[plo]")
-    L.append("s_mov_b32 s73, %[phi]")
+    # the batch (s36..s51) and the stream address (s72:s73) are the asm statement's in/out operands, bound to these very
+    # registers by their constraints: no copies in or out
     L.append("s_mov_b32 s70, 0xc000")
     for r in range(R):
         L.append("v_mov_b32 v%d, 0" % (c["a0"] + r))
@@ -181,10 +179,6 @@ def walk(nq, variant="", share=1):
     L.append("s_setprio 3")  # what follows a walk (issuing the staging loads, reaching the barrier) should not wait
     L.append("s_waitcnt lgkmcnt(0)")  # drain the look-ahead reads (their data is not used)
     L.append("s_set_gpr_idx_off")
-    for i in range(8):
-        L.append("s_mov_b64 %%[c%d], s[%d:%d]" % (i, 36 + 2 * i, 37 + 2 * i))
-    L.append("s_mov_b32 %[plo], s72")
-    L.append("s_mov_b32 %[phi], s73")
     return c, L
 
 
