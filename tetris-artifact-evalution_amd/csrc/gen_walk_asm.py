@@ -134,17 +134,22 @@ def walk(nq, variant="", share=1):
             if exits and r > 0:  # (a call is never made for an empty stream: the first entry of a batch is real)
                 L.append("s_cmp_eq_u32 s%d, 0" % (37 + 2 * r))
                 L.append("s_cbranch_scc1 8f")
-            if r == refill_at:
+            if r == refill_at and not exits:
                 # the next batch must have arrived; its addresses replace the ones all consumed by now
                 L.append("s_waitcnt lgkmcnt(0)")
                 L.extend(addresses(c, 52))
             la = r + ahead  # record whose reads are issued now
-            L.extend(reads(c, la % nbuf, c["a0"] + (la % R)))
+            # The last batch of a call reads nothing beyond itself (the next call forms its own addresses and primes
+            # its own reads), so its waits count only the reads of its later records; the scalar fetch of the next
+            # batch may still be in flight, which only makes such a wait stricter.
+            if not exits or la < R:
+                L.extend(reads(c, la % nbuf, c["a0"] + (la % R)))
+            in_flight = ahead if not exits else min(R - 1, la) - r
             for kk in range(share):
                 e = r * share + kk
                 L.append("s_lshr_b32 m0, s%d, 16" % (36 + 2 * e))
                 if kk == 0:
-                    L.append("s_waitcnt lgkmcnt(%d)" % (ahead * nq))
+                    L.append("s_waitcnt lgkmcnt(%d)" % (in_flight * nq))
                 else:
                     L.append("s_nop 0")  # keeps one instruction between the write of M0 and the indexed VALU use
                 L.extend(fmas(c, r % nbuf, 37 + 2 * e))
