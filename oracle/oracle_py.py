@@ -113,6 +113,38 @@ def ref_host_conv2d(x, w, stride, pad):
     return out
 
 
+def nchw_to_nhwc(x):
+    x = np.ascontiguousarray(x, np.float32)
+    n, c, h, w = x.shape
+    out = np.empty((n, h, w, c), np.float32)
+    _lib.orc_nchw_to_nhwc(x, out, n, c, h, w)
+    return out
+
+
+def nhwc_to_nchw(x):
+    x = np.ascontiguousarray(x, np.float32)
+    n, h, w, c = x.shape
+    out = np.empty((n, c, h, w), np.float32)
+    _lib.orc_nhwc_to_nchw(x, out, n, c, h, w)
+    return out
+
+
+def ref_nchw_to_nhwc(x):
+    """The reference's in-place NCHW2NHWC (tensor_utils.cc:85-108) on a copy."""
+    x = np.array(x, np.float32, order="C")
+    n, c, h, w = x.shape
+    _ref.ref_nchw2nhwc(x, n, c, h, w)
+    return x.reshape(n, h, w, c)
+
+
+def ref_nhwc_to_nchw(x):
+    """The reference's in-place NHWC2NCHW (tensor_utils.cc:110-134) on a copy."""
+    x = np.array(x, np.float32, order="C")
+    n, h, w, c = x.shape
+    _ref.ref_nhwc2nchw(x, n, c, h, w)
+    return x.reshape(n, c, h, w)
+
+
 def float_equal(a, b):
     return bool(_lib.orc_float_equal(a, b))
 

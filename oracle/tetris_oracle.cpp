@@ -397,7 +397,7 @@ int orc_read_weight_file(const char* path, int32_t* hdr, float** filter_out, int
 
 void orc_free(void* p) { free(p); }
 
-// tensor_utils.cc:85-97 / :99-111 (out of place here)
+// tensor_utils.cc:87-99 (NCHW2NHWC) / :101-113 (NHWC2NCHW); out of place here, the reference works in place
 void orc_nchw_to_nhwc(const float* src, float* dst, int N, int C, int H, int W) {
   for (int n = 0; n < N; ++n)
     for (int h = 0; h < H; ++h)

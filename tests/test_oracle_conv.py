@@ -93,6 +93,26 @@ def test_float_equal_predicate(oracle):
     assert oracle.tensor_first_mismatch(x, y) == 7
 
 
+def test_layout_transposes(oracle):
+    # tensor_utils.cc:85-134 (NCHW2NHWC / NHWC2NCHW): against numpy.transpose, as a round trip, on ragged extents and
+    # on an empty tensor, and against the reference's own in-place routines compiled as they lie
+    rng = np.random.default_rng(31)
+    for shape in [(1, 1, 1, 1), (2, 3, 5, 7), (3, 8, 4, 4), (1, 17, 2, 9), (2, 1, 6, 1), (0, 4, 3, 3)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        nhwc = oracle.nchw_to_nhwc(x)
+        assert nhwc.shape == (shape[0], shape[2], shape[3], shape[1])
+        assert np.array_equal(nhwc, np.transpose(x, (0, 2, 3, 1)))
+        back = oracle.nhwc_to_nchw(nhwc)
+        assert np.array_equal(back, x) and np.array_equal(back, np.transpose(nhwc, (0, 3, 1, 2)))
+        if oracle.ref_available() and x.size:
+            assert np.array_equal(oracle.ref_nchw_to_nhwc(x), nhwc)
+            assert np.array_equal(oracle.ref_nhwc_to_nchw(nhwc), x)
+    # a tensor whose value IS its NCHW index makes a swapped pair of axes visible element by element
+    x = np.arange(2 * 3 * 4 * 5, dtype=np.float32).reshape(2, 3, 4, 5)
+    nhwc = oracle.nchw_to_nhwc(x)
+    assert nhwc[1, 2, 3, 1] == x[1, 1, 2, 3] == 1 * 60 + 1 * 20 + 2 * 5 + 3
+
+
 def test_weight_reader_on_a_written_file(oracle, tmp_path):
     # header order H W IC OC KS PAD STRIDE GROUPS (tensor_utils.cc:66), then OC*IC*KS*KS floats, OIHW
     vals = np.array([0.0, -0.0, 1.5, -2.25e-3, 7, 1e-8, 0.0, 3.25], np.float32)
