@@ -289,22 +289,25 @@ def summary_line(full, details):
     rl = full["roofline"]
     line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
                                  "ms_per_step_device", "higher_is_better", "scaling", "vs_baseline", "dtype", "data")}
-    line["metric"] = "effective GFLOP/s (dense-equivalent) over the sparse conv layer stack"
+    line["metric"] = "effective GFLOP/s (dense-equivalent) of the sparse conv stack"
     line["config"] = pick(full["config"], ("workload", "suite", "batch", "layers"))
     line["check"] = None if full["check"] is None else pick(full["check"], (
-        "ok", "max_rel_err", "tolerance", "layers_checked", "all_workloads_ok", "failed_workloads"))
+        "ok", "max_rel_err", "tolerance", "all_workloads_ok") + (() if full["check"]["all_workloads_ok"] else ("failed_workloads",)))
     line["roofline"] = pick(rl, ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "avg_launch_us",
                                  "launches_per_step", "algorithmic_flops_per_launch", "algorithmic_bytes_per_launch"))
+    for k in ("algorithmic_flops_per_launch", "algorithmic_bytes_per_launch", "traffic"):
+        if line["roofline"].get(k) is not None:
+            line["roofline"][k] = int(round(line["roofline"][k]))
     line["roofline"]["note"] = rl.get("note")
     cpu = full["cpu_baseline"]
     line["cpu_baseline"] = None if cpu is None else pick(cpu, ("value", "unit", "cores", "kind", "sample"))
     line["min_layer_roofline_frac"] = full["min_layer_roofline_frac"]
     ctx = full["context"] or {}
-    line["context"] = pick(ctx, ("measured_copy_gbs", "measured_fma_tflops", "roofline_frac_of_measured",
-                                 "vendor_dense_fp32_ms_per_step", "vendor_csr_im2col_ms_per_step"))
+    line["context"] = pick(ctx, ("measured_copy_gbs", "measured_fma_tflops", "vendor_dense_fp32_ms_per_step",
+                                 "vendor_csr_im2col_ms_per_step"))
     # other workloads: [suite, batch, ms per pass, bound, fraction of the binding roof, smallest layer fraction,
     #                   counter bytes / algorithmic bytes, check ok]
-    line["suites_columns"] = "suite,batch,ms,bound,frac,min_layer_frac,traffic_ratio,check_ok"
+    line["suites_cols"] = "suite,batch,ms,bound,frac,min_layer_frac,traffic_ratio,check_ok"
     line["suites"] = [[r["suite"], r["batch"], r["ms_per_step_device"], r["bound"].replace("valu_", ""), r["roofline_frac"],
                        r["min_layer_roofline_frac"],
                        round(r["traffic"] / r["algorithmic_bytes_per_launch"], 3) if r.get("traffic") else None,
@@ -410,7 +413,7 @@ def main():
         achieved = fl_sparse / t_step / 1e12
         # the contract's label for the compute roof is "mfma"; the work here is vector fp32 FMA on the VALU, no MFMA
         roofline = {"bound": "mfma", "bound_detail": "valu_fp32",
-                    "note": "vector fp32 FMA on the VALU, no MFMA; 157.3 needs packed fp32 (compiled off: 78.6 reachable)",
+                    "note": "VALU fp32 FMA, no MFMA; the peak needs packed fp32 (compiled off here: 78.6 reachable)",
                     "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP32_TFLOPS, 4)}
     else:
@@ -472,8 +475,8 @@ def main():
                 break
         cpu = {"value": round(done_fl / t_cpu / 1e9, 2), "unit": "GFLOP/s", "cores": threads,
                "kind": "port", "sample": "first %d of %d %s layers, batch %d, one pass: reference SparseFilter layout (TILE_IC 32, "
-               "Bank-SR + ReorderOutChannel, vec4) decoded by the oracle's HostReorderSpconv2d restatement, OpenMP over "
-               "(n, oc), %.1f s" % (used, len(layers), args.suite, N, t_cpu),
+               "Bank-SR + ReorderOutChannel, vec4) decoded by the oracle's HostReorderSpconv2d, OpenMP over (n, oc), %.1f s"
+               % (used, len(layers), args.suite, N, t_cpu),
                "pack_s": round(t_cpu_pack, 2),
                "gpu_vs_this_cpu_output_max_rel_err": None if args.no_check else agree}
         if not args.no_check and not agree <= 1e-4:
@@ -560,7 +563,7 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "ms_per_step_device": round(ms_per_step_dev, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "%s-shaped sparse conv stack, %d layers, batch %d, fp32 NCHW, seeded unstructured masks"
+        "config": {"workload": "%s-shaped sparse conv stack, %d layers, batch %d, fp32 NCHW, seeded masks"
                    % (args.suite, len(layers), N), "suite": args.suite, "batch": N, "layers": len(layers),
                    "base_seed": W.BASE_SEED,
                    "tensor_seed": "base_seed ^ crc32('<suite>/<layer index>/<w|x>'), splitmix64 streams "

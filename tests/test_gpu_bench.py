@@ -48,7 +48,7 @@ def test_default_command_prints_one_short_line():
     lines = r.stdout.strip().splitlines()
     assert len(lines) == 1, [ln[:80] for ln in lines]
     line = lines[-1]
-    assert len(line) < 4096, len(line)
+    assert len(line) < 2000, len(line)  # a reader that keeps the last 2000 characters of stdout holds the whole line
     d = json.loads(line)
     assert d["n_gpus"] == 1 and d["steps"] == 5 and d["warmup"] == 2 and d["config"]["suite"] == "vgg19"
     assert d["config"]["batch"] == 16 and d["check"]["ok"] and d["check"]["all_workloads_ok"], d["check"]
@@ -58,7 +58,7 @@ def test_default_command_prints_one_short_line():
     assert len(d["suites"]) == 7 and all(row[-1] is True for row in d["suites"]), d["suites"]
     assert d["chain"]["check_ok"] is True
     full = json.load(open(os.path.join(ROOT, d["details"])))
-    assert len(full["layers"]) == 16 and sum(len(s["layers"]) for s in full["suites"]) == 174
+    assert len(full["layers"]) == 16 and sum(len(s["layers"]) for s in full["suites"]) == 190
 
 
 def test_summary_line_stays_short():
@@ -87,7 +87,7 @@ def test_summary_line_stays_short():
                         "peaks_note": "p" * 300},
             "suites": suites, "chain": {"ms_per_pass": 2.0845, "check": {"ok": True}, "workload": "c" * 300}}
     line = json.dumps(bench.summary_line(full, os.path.join(ROOT, "gpurun_out", "bench_layers.json")))
-    assert len(line) < 3000, len(line)
+    assert len(line) < 2400, len(line)
     d = json.loads(line)
     for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline", "check"):
