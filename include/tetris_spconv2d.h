@@ -141,6 +141,10 @@ int tetris_tile_table_load(const char* path, int* rows_out);
  * finds its input, its weights and its code in HBM, and the tile that wins from warm caches, as back-to-back launches
  * of one layer measure it (the reference's protocol, Tetris/spconv2d.cc:44-68), is not always the one that wins there. */
 #define TETRIS_OPT_COLD_TIMING 4u
+/* tetris_spconv2d_launch_spf / _spf_arrays take a set of device arrays they have already decoded once as unchanged:
+ * no read-back, no hash, no synchronisation -- the launch is then as asynchronous as tetris_spconv2d_launch.  A caller
+ * that rewrites the arrays in place says so with tetris_spf_invalidate. */
+#define TETRIS_OPT_TRUST_SPF_ARRAYS 8u
 int tetris_options_set(unsigned flags);
 unsigned tetris_options_get(void);
 
@@ -247,13 +251,24 @@ size_t tetris_noalloc_scratch_limit(size_t bytes);
  * out).  d_stage_len is accepted and not read, as in the reference's kernel.  tile_ic and vec_width are the
  * SparseFilter's TILE_IC (a template argument of the reference launcher) and entries per lane and step: 4
  * (apply_vectorize), 1, or 0 for the keep-as-is layout of apply_reorder = false (spconv2d_utils.h:38-61; then
- * d_oc_permutation may be NULL) -- the format of the reference's CSR-like baseline variant.  tile: NULL = the library
- * chooses.  Not capturable into a HIP graph (it synchronises); capture tetris_spconv2d_launch instead. */
+ * d_oc_permutation may be NULL) -- the format of the reference's CSR-like baseline variant.  n_entries: how many
+ * entries d_position and d_values hold (0: not known).  Before any kernel reads the arrays the offsets are copied to
+ * the host and checked -- they start at 0, never decrease, step by multiples of vec_width and span at most n_entries
+ * entries -- so a wrong out_channel, tile_ic or vec_width is TETRIS_EINVAL, not an out-of-range read on the device.
+ * tile: NULL = the library chooses.  Not capturable into a HIP graph (it synchronises); capture
+ * tetris_spconv2d_launch instead.  With TETRIS_OPT_TRUST_SPF_ARRAYS a set of arrays seen before is neither read back
+ * nor hashed (see there). */
 int tetris_spconv2d_launch_spf_arrays(const float* d_input, const int32_t* d_offsets, const int32_t* d_stage_len,
                                       const int32_t* d_oc_permutation, const int32_t* d_position, const float* d_values,
                                       float* d_output, int batch, int img_h, int img_w, int in_channel, int out_channel,
                                       int kernel_size, int stride, int padding, int tile_ic, int vec_width,
-                                      const tetris_tile* tile, void* stream);
+                                      int64_t n_entries, const tetris_tile* tile, void* stream);
+/* Forgets what the two launchers above remember about the arrays whose values live at d_values: the next call decodes
+ * them again.  For callers that rewrite the arrays in place under TETRIS_OPT_TRUST_SPF_ARRAYS. */
+void tetris_spf_invalidate(const float* d_values);
+/* The host-side check the launchers apply to a copy of d_offsets, usable on its own: n_offsets =
+ * ceil(out_channel / 32) * stages + 1 (out_channel * stages + 1 for vec_width 0).  TETRIS_OK or TETRIS_EINVAL. */
+int tetris_spf_check_offsets(const int32_t* h_offsets, int64_t n_offsets, int vec_width, int64_t n_entries);
 
 /* Same, in the exact call shape of the reference launcher, which carries neither TILE_IC nor the vector width:
  * those two are taken from the live tetris_spf whose device arrays these are (found through d_values;
@@ -288,7 +303,10 @@ int tetris_spconv2d_spf_host(const float* h_input, const float* h_filter, float*
 /* Replaces SparseConv2d_Baseline<float,int,int> (Tetris/baseline.cc:22-93), the first rung of the reference's
  * ablation ladder: as tetris_spconv2d_spf_host, but the SparseFilter is built with apply_reorder = false (baseline.cc:44:
  * the keep-as-is, CSR-like arrays of spconv2d_utils.h:38-61, no channel permutation) and those arrays feed the
- * convolution (tetris_spconv2d_launch_spf_arrays with vec_width 0), run with the same fixed tile. */
+ * convolution (tetris_spconv2d_launch_spf_arrays with vec_width 0), run with the same fixed tile at ONE output
+ * channel per wave: every wave walks one stream per (output channel, stage) in file order, as a thread of the
+ * reference's baseline kernel walks one run per (output channel, stage) (Tetris/ablation_kernel.cu:76-98); no
+ * channels are merged into a stream and no channel order is chosen.  That is the step "Baseline -> SPF" measures. */
 int tetris_spconv2d_baseline_host(const float* h_input, const float* h_filter, float* h_output, int batch, int img_h,
                                   int img_w, int in_channel, int out_channel, int kernel_size, int stride, int padding,
                                   void* stream, const char* layout, float* ms_out);

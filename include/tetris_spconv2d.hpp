@@ -121,7 +121,7 @@ void SparseConv2d(ValueType* input, OffsetType* offsets, OffsetType* stage_len, 
     TETRIS_CHECK(tetris_spconv2d_launch_spf_arrays(
         input, reinterpret_cast<const int32_t*>(offsets), reinterpret_cast<const int32_t*>(stage_len),
         reinterpret_cast<const int32_t*>(oc_permutation), reinterpret_cast<const int32_t*>(position), values, output,
-        batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding, TILE_IC, 4, nullptr,
+        batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding, TILE_IC, 4, /*n_entries unknown*/ 0, nullptr,
         reinterpret_cast<void*>(stream)));
   else
     TETRIS_CHECK(tetris_spconv2d_launch_spf(input, reinterpret_cast<const int32_t*>(offsets),

@@ -23,7 +23,8 @@ def _load(path):
     return C.CDLL(path)
 
 
-_lib = _load(os.path.join(_HERE, "libtetris_oracle.so"))
+# TETRIS_ORACLE_LIB: another build of the oracle (the sanitizer build of `make asan`)
+_lib = _load(os.environ.get("TETRIS_ORACLE_LIB") or os.path.join(_HERE, "libtetris_oracle.so"))
 _ref = _load(os.path.join(_HERE, "_ref", "libtetris_ref.so"))
 
 

@@ -3,8 +3,9 @@
 * weights_*.npz   five shipped pruned layers, parsed by the reference's own ReadConfigAndDataFromFile
                   (tensor_utils.cc:55-82, compiled unmodified into oracle/_ref) -- data files, stored as float32
                   arrays plus the eight header ints.
-* masks_*.npz     the zero patterns of every shipped layer of two pruned networks (VGG19 at 92 %, MobileNetV1 at
-                  86 %): per layer the eight header ints and numpy.packbits(weight != 0), plus the file names.
+* masks_*.npz     the zero patterns of every shipped layer of five pruned networks (VGG19 at 92 %, MobileNetV1 at
+                  86 %, ResNet-50 at 90 % and at 98 %, YOLOv3 at 89 %, the loop of evalution/conv2d_timing.py:136-176):
+                  per layer the eight header ints and numpy.packbits(weight != 0), plus the file names.
                   tetris_amd.workloads.pruned_suite() turns them into benchmark layers with seeded values.
 * spf_known_answers.json is NOT produced here: it is the table of FNV-1a-64 hashes and array sizes that was
   recorded from the compiled reference SparseFilter (spconv2d_utils.h) for these layers; the reference's CUDA
@@ -36,7 +37,9 @@ BIG_FILES = {
     "vgg_256": "vgg19/vgg19-92-acc-71.7/module8_0_module2_0_conv2d_3_H_56_W_56_IC_256_OC_256_KS_3_Pad_1_S_1_G_1",
 }
 
-MASK_DIRS = {"vgg19_92": "vgg19/vgg19-92-acc-71.7", "mobilenet_86": "mobilenet/mobilenet-86-acc-70.1"}
+MASK_DIRS = {"vgg19_92": "vgg19/vgg19-92-acc-71.7", "mobilenet_86": "mobilenet/mobilenet-86-acc-70.1",
+             "resnet50_90": "resnet50/ResNet50-magnitude-90-acc-73.91", "resnet50_98": "resnet50/ResNet50-magnitude-98-acc-57.90",
+             "yolov3_89": "yolov3/yolov3-89-acc-62.4"}
 
 
 def write_masks(tag, rel):

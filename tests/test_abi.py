@@ -170,7 +170,9 @@ def test_balanced_order_rejects_bad_arguments():
         T.oc_order_balanced(w, T.Tile(7, 2, 0, 8, 8))
 
 
-@pytest.mark.parametrize("masks,count", [("masks_vgg19_92.npz", 8), ("masks_mobilenet_86.npz", 13)])
+@pytest.mark.parametrize("masks,count", [("masks_vgg19_92.npz", 8), ("masks_mobilenet_86.npz", 13),
+                                         ("masks_resnet50_90.npz", 44), ("masks_resnet50_98.npz", 44),
+                                         ("masks_yolov3_89.npz", 55)])
 def test_pruned_suites_load_and_balance(masks, count):
     from tetris_amd import workloads as W
 
@@ -190,6 +192,51 @@ def test_pruned_suites_load_and_balance(masks, count):
         bal, _ = _busiest_wave_cost(w, order, tile.oc_per_wave, tile.waves, tile.tile_ic)
         gains.append(bal / ident)
     assert max(gains) <= 1.0 and np.mean(gains) <= 0.93, gains
+
+
+def test_host_packer_on_negative_zeros_and_denormals(oracle):
+    # `value != 0.f` (Tetris/spconv2d_utils.h:47, :87): -0.0 is dropped, a denormal is kept -- in all four flag sets
+    rng = np.random.default_rng(17)
+    w = sparse_filter(rng, 40, 24, 3, 0.7, neg_zero=True)
+    flat = w.reshape(-1)
+    nz = np.flatnonzero(flat)
+    flat[nz[::4]] = np.float32(1e-40)
+    flat[nz[1::4]] = np.float32(-1.4e-45)
+    assert np.signbit(flat[flat == 0]).any()
+    for flags in (0, 1, 2, 3):
+        sf = T.SparseFilter(w, 24, 40, 3, 16, True, True, flags)
+        ref = oracle.SpfPack(w, 16, True, True, bool(flags & 1), bool(flags & 2))
+        assert sf.values_.tobytes() == ref.values.tobytes() and np.array_equal(sf.position_, ref.position)
+        assert int((sf.values_ != 0).sum()) == int((w != 0).sum())            # every denormal packed, no zero packed
+        assert not (sf.values_.view(np.uint32) == 0x80000000).any()           # -0.0 never stored
+        sf.close()
+    sf = T.SparseFilter(w, 24, 40, 3, 16, False, True, 0)
+    assert sf.nnz_ == int((w != 0).sum())
+    sf.close()
+
+
+def test_offsets_check_of_the_raw_launchers(oracle):
+    # What the raw launchers verify on a host copy of offsets_ before any kernel reads the arrays
+    # (Tetris/spconv2d_utils.h:45-47, 209-216: starts at 0, never decreases, steps of the vector width)
+    rng = np.random.default_rng(5)
+    w = sparse_filter(rng, 70, 40, 3, 0.8)
+    for vec, args in [(4, (True, True, True, True)), (1, (True, False, True, True)), (0, (False,))]:
+        p = oracle.SpfPack(w, 16, *args)
+        off, n_ent = p.offsets, len(p.values)
+        T.spf_check_offsets(off, vec, n_ent)
+        T.spf_check_offsets(off, vec, 0)  # capacity not known
+        for bad, cap in [(off, n_ent - 1), (off[::-1], n_ent), (off + 1, n_ent), (-off, n_ent)]:
+            with pytest.raises(T.TetrisError) as e:
+                T.spf_check_offsets(bad, vec, cap)
+            assert e.value.code == T.EINVAL
+    p = oracle.SpfPack(w, 16, True, True, True, True)
+    odd = p.offsets.copy()
+    odd[1:] += 2
+    with pytest.raises(T.TetrisError):
+        T.spf_check_offsets(odd, 4, 0)
+    T.spf_check_offsets(odd - np.where(np.arange(len(odd)) > 0, 2, 0), 4, 0)
+    with pytest.raises(T.TetrisError):
+        T.spf_check_offsets(p.offsets, 3, 0)  # no such vector width
 
 
 def test_tile_table_loaded_at_run_time_wins_over_the_built_in_one(tmp_path):

@@ -245,28 +245,20 @@ void drop_views(const void* d_values) {
 }
 
 // The kernel pack (and tile) for a convolution whose weights are the arrays at these addresses, rebuilt when the
-// arrays' content has changed since the view was made.  Hashing reads the arrays once and synchronises `stream`.
+// arrays' content has changed since the view was made.  The caller holds g_views_mu, and keeps it until the launch
+// that uses the pack has been issued: a view (and its packs) can only be evicted or dropped under that lock.
+// Before any kernel touches the arrays the offsets are copied to the host and checked (non-negative, non-decreasing,
+// the entries they span within `capacity` when the caller gave one), so that a wrong K, tile_ic or vector width is
+// an error code and not an out-of-bounds read on the device.  Hashing reads the arrays once and synchronises `stream`;
+// with TETRIS_OPT_TRUST_SPF_ARRAYS a view that exists for these addresses is used as it is (no read-back, no
+// synchronisation) until tetris_spf_invalidate or tetris_spf_destroy drops it.
 int view_pack(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_position, const float* d_values, int N,
-              int H, int W, int C, int K, int ks, int stride, int pad, int tile_ic, int vec, const tetris_tile* tile,
-              hipStream_t stream, tetris_g950** pack_out, tetris_tile* tile_out) {
+              int H, int W, int C, int K, int ks, int stride, int pad, int tile_ic, int vec, long long capacity,
+              const tetris_tile* tile, hipStream_t stream, tetris_g950** pack_out, tetris_tile* tile_out) {
   if (!d_offsets || !d_position || !d_values || (vec != 0 && !d_perm)) return fail(TETRIS_EINVAL, "null argument");
   if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || tile_ic <= 0 || (vec != 0 && vec != 1 && vec != 4))
     return fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d tile_ic=%d vector width=%d", C, K, ks, tile_ic, vec);
-  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
-    return fail(TETRIS_EINVAL, "this entry point reads the arrays back (a synchronisation): it cannot be captured; "
-                "capture tetris_spconv2d_launch on a tetris_g950 instead");
-  const int stages = (C - 1) / tile_ic + 1;
-  const int n_off = (vec == 0 ? K : (K + kRefLanes - 1) / kRefLanes) * stages + 1;
-  std::lock_guard<std::mutex> lock(g_views_mu);
-  if (!g_hash_scratch) TETRIS_HIP(hipMalloc(&g_hash_scratch, 16));
-  unsigned long long hash = 0;
-  long long n_ent = 0;
-  int rc = spf_arrays_hash(d_offsets, n_off, d_perm, vec == 0 ? 0 : K, d_position, d_values, vec == 0 ? 1 : kRefLanes,
-                           g_hash_scratch, stream, &hash, &n_ent);
-  if (rc) return rc;
-  if (n_ent < 0 || n_ent > (1ll << 31)) return fail(TETRIS_EINVAL, "offsets end at %lld entries: not a packed filter", n_ent);
-  hash ^= 0x5bd1e995ull * (unsigned long long)(C * 131 + ks) + (unsigned long long)tile_ic * 7919ull + (unsigned)vec;
+  if (capacity < 0) return fail(TETRIS_EINVAL, "negative entry capacity");
   SpfView* v = nullptr;
   for (size_t i = 0; i < g_views.size(); ++i) {
     SpfView* c = g_views[i];
@@ -275,6 +267,42 @@ int view_pack(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_
       v = c;
       g_views.erase(g_views.begin() + (long)i);
       break;
+    }
+  }
+  const bool trusted = v && v->d_filter && (options() & TETRIS_OPT_TRUST_SPF_ARRAYS);
+  unsigned long long hash = v ? v->hash : 0;
+  int rc = TETRIS_OK;
+  if (!trusted) {
+    if (v) g_views.push_back(v);  // stays registered whatever the checks below say
+    v = nullptr;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return fail(TETRIS_EINVAL, "this entry point reads the arrays back (a synchronisation): it cannot be captured; "
+                  "capture tetris_spconv2d_launch on a tetris_g950 instead");
+    const int stages = (C - 1) / tile_ic + 1;
+    const long long n_off_ll = (long long)(vec == 0 ? K : (K + kRefLanes - 1) / kRefLanes) * stages + 1;
+    if (n_off_ll > (1ll << 28)) return fail(TETRIS_EINVAL, "%lld stream offsets: not a packed filter", n_off_ll);
+    const int n_off = (int)n_off_ll;
+    const int lanes = vec == 0 ? 1 : kRefLanes;
+    std::vector<int32_t> h_off((size_t)n_off);
+    TETRIS_HIP(hipMemcpyAsync(h_off.data(), d_offsets, sizeof(int32_t) * (size_t)n_off, hipMemcpyDeviceToHost, stream));
+    TETRIS_HIP(hipStreamSynchronize(stream));
+    rc = check_spf_offsets(h_off.data(), n_off, lanes, vec, capacity);
+    if (rc) return rc;
+    const long long n_ent = (long long)lanes * h_off[n_off - 1];
+    if (!g_hash_scratch) TETRIS_HIP(hipMalloc(&g_hash_scratch, 16));
+    rc = spf_arrays_hash(d_offsets, n_off, d_perm, vec == 0 ? 0 : K, d_position, d_values, n_ent, g_hash_scratch, stream,
+                         &hash);
+    if (rc) return rc;
+    hash ^= 0x5bd1e995ull * (unsigned long long)(C * 131 + ks) + (unsigned long long)tile_ic * 7919ull + (unsigned)vec;
+    for (size_t i = 0; i < g_views.size(); ++i) {
+      SpfView* c = g_views[i];
+      if (c->ptrs[0] == d_offsets && c->ptrs[1] == d_perm && c->ptrs[2] == d_position && c->ptrs[3] == d_values &&
+          c->C == C && c->K == K && c->ks == ks && c->tile_ic == tile_ic && c->vec == vec) {
+        v = c;
+        g_views.erase(g_views.begin() + (long)i);
+        break;
+      }
     }
   }
   if (!v) {
@@ -354,12 +382,27 @@ tetris_tile fixed_spf_tile(int N, int H, int W, int C, int K, int ks, int stride
   return t;
 }
 
+// The Baseline rung's tile: the fixed tile with ONE output channel per wave, so that a wave walks one stream per (output
+// channel, stage) in file order -- the keep-as-is runs of the CSR-like arrays, no channels grouped into a stream and
+// no channel order chosen -- where the SPF rung's waves walk the merged, position-sorted stream of eight channels.
+tetris_tile baseline_tile(tetris_tile t, int N, int H, int W, int C, int K, int ks, int stride, int pad) {
+  tetris_tile b = t;
+  b.oc_per_wave = 1;
+  tetris_g950 shape;
+  shape.C = C; shape.K = K; shape.ks = ks; shape.tile_ic = b.tile_ic; shape.g = b.oc_per_wave;
+  shape.stages = ceil_div(C, b.tile_ic);
+  shape.slots = ceil_div(K, kSlotPad) * kSlotPad;
+  Geom g;
+  return make_geom(&shape, N, H, W, stride, pad, b, &g) == TETRIS_OK ? b : t;
+}
+
 // Shared body of the two host-to-host entry points.  spf_path: the reference's SparseConv2d_SPF (Tetris/spf.cc:22-93):
 // SparseFilter with TILE_IC = 128 and apply_reorder = true whatever the caller passed (:43-44), its device arrays handed
 // to the launcher, one fixed tile.
 // baseline: the reference's SparseConv2d_Baseline (Tetris/baseline.cc:22-93): SparseFilter with TILE_IC = 128 and
 // apply_reorder = false (the keep-as-is, CSR-like arrays of spconv2d_utils.h:38-61) handed to the launcher, the same
-// fixed tile.
+// fixed tile with one output channel per wave (baseline_tile): one stream per (output channel, stage), as the
+// reference's baseline kernel walks one run per (thread = output channel, stage) (ablation_kernel.cu:76-98).
 int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int H, int W, int C, int K, int ks,
               int stride, int pad, hipStream_t stream, bool apply_reorder, bool spf_path, unsigned spf_flags,
               float* ms_out, bool baseline = false) {
@@ -373,7 +416,9 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
   tetris_spf* spf = nullptr;     // owned here (the spf path; its view owns the pack)
   float *d_in = nullptr, *d_out = nullptr;
   const size_t in_bytes = sizeof(float) * (size_t)N * C * H * W, out_bytes = sizeof(float) * (size_t)N * K * OH * OW;
+  std::unique_lock<std::mutex>* held = nullptr;
   auto done = [&](int code) {
+    if (held && held->owns_lock()) held->unlock();  // tetris_spf_destroy drops the views under the same lock
     if (d_in) (void)hipFree(d_in);
     if (d_out) (void)hipFree(d_out);
     tetris_g950_destroy(pack);
@@ -382,15 +427,20 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
   };
   int rc;
   tetris_g950* run = nullptr;
+  // the spf path runs on a pack its view owns: the views' lock is held until the launches have been issued
+  std::unique_lock<std::mutex> views_lock(g_views_mu, std::defer_lock);
+  held = &views_lock;
   if (spf_path) {
     rc = tetris_spf_create(h_filter, C, K, ks, 128, baseline ? 0 : 1, 1, spf_flags, &spf);
     if (rc) return done(rc);
     tetris_spf_arrays a{};
     rc = tetris_spf_device_arrays(spf, &a);
     if (rc) return done(rc);
-    const tetris_tile fixed = fixed_spf_tile(N, H, W, C, K, ks, stride, pad);
+    tetris_tile fixed = fixed_spf_tile(N, H, W, C, K, ks, stride, pad);
+    if (baseline) fixed = baseline_tile(fixed, N, H, W, C, K, ks, stride, pad);
+    views_lock.lock();
     rc = view_pack(a.offsets, baseline ? nullptr : a.oc_permutation, a.position, a.values, N, H, W, C, K, ks, stride, pad,
-                   128, baseline ? 0 : 4, &fixed, stream, &run, &tile);
+                   128, baseline ? 0 : 4, a.n_values, &fixed, stream, &run, &tile);
     if (rc) return done(rc);
   } else {
     rc = choose_tile(N, H, W, C, K, ks, stride, pad, &tile);
@@ -419,6 +469,7 @@ int conv_host(const float* h_in, const float* h_filter, float* h_out, int N, int
   HIPD(hipMemcpyAsync(d_in, h_in, in_bytes, hipMemcpyHostToDevice, stream));
   float ms = 0;
   rc = time_launches(run, d_in, d_out, N, H, W, stride, pad, &tile, stream, 30, 100, &ms);
+  if (views_lock.owns_lock()) views_lock.unlock();
   if (rc) return done(rc);
   HIPD(hipMemcpyAsync(h_out, d_out, out_bytes, hipMemcpyDeviceToHost, stream));
   HIPD(hipStreamSynchronize(stream));
@@ -517,7 +568,7 @@ int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* o) {
 }
 
 int tetris_options_set(unsigned flags) {
-  if (flags & ~(TETRIS_OPT_PAIRS | TETRIS_OPT_NO_BANK_RULE | TETRIS_OPT_COLD_TIMING))
+  if (flags & ~(TETRIS_OPT_PAIRS | TETRIS_OPT_NO_BANK_RULE | TETRIS_OPT_COLD_TIMING | TETRIS_OPT_TRUST_SPF_ARRAYS))
     return fail(TETRIS_EINVAL, "unknown option bits 0x%x", flags);
   set_options(flags);
   return TETRIS_OK;
@@ -702,16 +753,21 @@ int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_in, float* d_o
 int tetris_spconv2d_launch_spf_arrays(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,
                                       const int32_t* d_perm, const int32_t* d_position, const float* d_values,
                                       float* d_out, int N, int H, int W, int C, int K, int ks, int stride, int pad,
-                                      int tile_ic, int vec_width, const tetris_tile* tile, void* stream_) {
+                                      int tile_ic, int vec_width, int64_t n_entries, const tetris_tile* tile,
+                                      void* stream_) {
   (void)d_stage_len;  // the reference's kernel does not read it either (Tetris/spconv2d_kernel.cu:13-160)
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   tetris_g950* pack = nullptr;
   tetris_tile t{};
-  int rc = view_pack(d_offsets, d_perm, d_position, d_values, N, H, W, C, K, ks, stride, pad, tile_ic, vec_width, tile, stream,
-                     &pack, &t);
+  // held until the launch is issued: the pack belongs to a view that another thread's call may evict or drop
+  std::lock_guard<std::mutex> lock(g_views_mu);
+  int rc = view_pack(d_offsets, d_perm, d_position, d_values, N, H, W, C, K, ks, stride, pad, tile_ic, vec_width,
+                     (long long)n_entries, tile, stream, &pack, &t);
   if (rc) return rc;
   return run_launch(pack, d_in, d_out, N, H, W, stride, pad, &t, stream);
 }
+
+void tetris_spf_invalidate(const float* d_values) { drop_views(d_values); }
 
 int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, const int32_t* d_stage_len,
                                const int32_t* d_perm, const int32_t* d_position, const float* d_values, float* d_out,
@@ -719,6 +775,7 @@ int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, cons
   // the call shape of the reference launcher carries neither TILE_IC (a template argument there) nor the vector
   // width: they are taken from the live tetris_spf that owns `d_values`; the CONTENT comes from the arrays
   int tile_ic = 0, vec = 0;
+  int64_t n_entries = 0;
   {
     std::lock_guard<std::mutex> lock(g_registry_mu);
     auto it = g_registry.find(d_values);
@@ -731,9 +788,10 @@ int tetris_spconv2d_launch_spf(const float* d_in, const int32_t* d_offsets, cons
                   f->K, f->ks);
     tile_ic = f->tile_ic;
     vec = f->vec;
+    n_entries = (int64_t)f->values.size();
   }
   return tetris_spconv2d_launch_spf_arrays(d_in, d_offsets, d_stage_len, d_perm, d_position, d_values, d_out, N, H, W, C,
-                                           K, ks, stride, pad, tile_ic, vec, nullptr, stream);
+                                           K, ks, stride, pad, tile_ic, vec, n_entries, nullptr, stream);
 }
 
 int tetris_spconv2d_time(tetris_g950* p, const float* d_in, float* d_out, int N, int H, int W, int stride, int pad,

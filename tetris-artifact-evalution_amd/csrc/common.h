@@ -216,15 +216,18 @@ namespace tetris {
 int spf_pack_host(const float* filter, int C, int K, int ks, int tile_ic, bool apply_reorder, bool apply_vectorize,
                   unsigned flags, tetris_spf* out);
 
+int check_spf_offsets(const int32_t* offsets, int n_off, int lanes, int vec, long long capacity);
+
 // spf_pack_device.hip
 // entries of the pack bound to geometry `g`; paired: rearranged into pairs and singles (kernels that walk pairs)
 int g950_bind(tetris_g950* p, const Geom& g, bool paired, hipStream_t stream, const int2** entries_out,
               const int32_t** grp_off_out, const int32_t** grp_pair_out, int* heads_off_out);
 
 // spf_pack_device.hip: the reference layout's device arrays as the source of a convolution
+// n_ent: entries of d_position / d_values to hash (the caller has read and checked the offsets on the host)
 int spf_arrays_hash(const int32_t* d_offsets, int n_off, const int32_t* d_perm, int K, const int32_t* d_position,
-                    const float* d_values, int lanes, unsigned long long* d_scratch2, hipStream_t stream,
-                    unsigned long long* hash_out, long long* n_ent_out);
+                    const float* d_values, long long n_ent, unsigned long long* d_scratch2, hipStream_t stream,
+                    unsigned long long* hash_out);
 int spf_arrays_decode(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_position, const float* d_values,
                       float* d_filter, int C, int K, int ks, int tile_ic, int vec, hipStream_t stream);
 

@@ -377,13 +377,12 @@ __device__ __forceinline__ unsigned long long mix64(unsigned long long z) {
   return z ^ (z >> 31);
 }
 
-// out[0] += order-independent hash of (array id, index, word) over the four arrays; out[1] = entry count
+// out[0] += order-independent hash of (array id, index, word) over the four arrays, n_ent entries of the last two
 __global__ __launch_bounds__(256) void spf_hash_kernel(const int32_t* __restrict__ offsets, int n_off,
                                                        const int32_t* __restrict__ perm, int K,
                                                        const int32_t* __restrict__ position,
-                                                       const float* __restrict__ values, int lanes,
+                                                       const float* __restrict__ values, long long n_ent,
                                                        unsigned long long* __restrict__ out) {
-  const long long n_ent = (long long)lanes * offsets[n_off - 1];
   const long long total = n_off + K + 2 * n_ent;
   unsigned long long h = 0;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
@@ -396,7 +395,6 @@ __global__ __launch_bounds__(256) void spf_hash_kernel(const int32_t* __restrict
   }
   for (int off = 32; off > 0; off >>= 1) h += __shfl_xor(h, off);
   if ((threadIdx.x & 63) == 0) atomicAdd(out, h);
-  if (blockIdx.x == 0 && threadIdx.x == 0) out[1] = (unsigned long long)n_ent;
 }
 
 // vec > 0: the reorder path's layout (Tetris/spconv2d_utils.h:206-244): one workgroup per (32-lane group, stage);
@@ -410,7 +408,7 @@ __global__ __launch_bounds__(256) void spf_decode_kernel(const int32_t* __restri
                                                          int C, int K, int ks, int tile_ic, int stages, int vec) {
   const int seg = blockIdx.x;
   const int stage = seg % stages, row = seg / stages;  // row: 32-lane group, or output channel when vec == 0
-  const int beg = offsets[seg], len = offsets[seg + 1] - beg;
+  const int beg = offsets[seg], len = max(offsets[seg + 1] - beg, 0);
   const int kk = ks * ks;
   if (vec == 0) {
     for (int e = threadIdx.x; e < len; e += blockDim.x) {
@@ -441,17 +439,16 @@ __global__ void fill_zero_kernel(float* __restrict__ p, long long n) {
 }  // namespace
 
 int spf_arrays_hash(const int32_t* d_offsets, int n_off, const int32_t* d_perm, int K, const int32_t* d_position,
-                    const float* d_values, int lanes, unsigned long long* d_scratch2, hipStream_t stream,
-                    unsigned long long* hash_out, long long* n_ent_out) {
+                    const float* d_values, long long n_ent, unsigned long long* d_scratch2, hipStream_t stream,
+                    unsigned long long* hash_out) {
   hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(64), 0, stream, reinterpret_cast<float*>(d_scratch2), 4ll);
   hipLaunchKernelGGL(spf_hash_kernel, dim3(256), dim3(256), 0, stream, d_offsets, n_off, d_perm, K, d_position, d_values,
-                     lanes, d_scratch2);
+                     n_ent, d_scratch2);
   TETRIS_HIP(hipGetLastError());
   unsigned long long h[2] = {0, 0};
   TETRIS_HIP(hipMemcpyAsync(h, d_scratch2, sizeof h, hipMemcpyDeviceToHost, stream));
   TETRIS_HIP(hipStreamSynchronize(stream));
   *hash_out = h[0];
-  *n_ent_out = (long long)h[1];
   return TETRIS_OK;
 }
 

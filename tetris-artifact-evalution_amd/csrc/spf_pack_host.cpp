@@ -321,4 +321,32 @@ int spf_pack_host(const float* filter, int C, int K, int ks, int T, bool apply_r
   return TETRIS_OK;
 }
 
+// What the device code that reads a SparseFilter's arrays relies on: offsets_ starts at 0 and never decreases
+// (spconv2d_utils.h:45-47, :213-216), every step of the interleaved layout is a multiple of the vector width (:209-212),
+// and the entries the offsets span -- `lanes` per unit of offset -- fit the arrays (`capacity` entries; 0: not known).
+int check_spf_offsets(const int32_t* offsets, int n_off, int lanes, int vec, long long capacity) {
+  if (!offsets || n_off < 1) return fail(TETRIS_EINVAL, "no offsets");
+  if (offsets[0] != 0) return fail(TETRIS_EINVAL, "offsets[0] is %d, not 0: not a packed filter", offsets[0]);
+  for (int i = 1; i < n_off; ++i) {
+    if (offsets[i] < offsets[i - 1])
+      return fail(TETRIS_EINVAL, "offsets decrease at %d (%d after %d): wrong out_channel, tile_ic or vector width?", i,
+                  offsets[i], offsets[i - 1]);
+    if (vec > 1 && (offsets[i] - offsets[i - 1]) % vec != 0)
+      return fail(TETRIS_EINVAL, "stream %d holds %d steps, not a multiple of the vector width %d", i - 1,
+                  offsets[i] - offsets[i - 1], vec);
+  }
+  const long long n_ent = (long long)lanes * offsets[n_off - 1];
+  if (n_ent > (1ll << 31)) return fail(TETRIS_EINVAL, "offsets end at %lld entries: not a packed filter", n_ent);
+  if (capacity > 0 && n_ent > capacity)
+    return fail(TETRIS_EINVAL, "offsets span %lld entries, the arrays hold %lld: wrong out_channel, tile_ic or vector width?",
+                n_ent, capacity);
+  return TETRIS_OK;
+}
+
 }  // namespace tetris
+
+extern "C" int tetris_spf_check_offsets(const int32_t* h_offsets, int64_t n_offsets, int vec_width, int64_t n_entries) {
+  if (n_offsets < 1 || n_offsets > (1ll << 28) || (vec_width != 0 && vec_width != 1 && vec_width != 4) || n_entries < 0)
+    return tetris::fail(TETRIS_EINVAL, "bad argument");
+  return tetris::check_spf_offsets(h_offsets, (int)n_offsets, vec_width == 0 ? 1 : tetris::kRefLanes, vec_width, n_entries);
+}

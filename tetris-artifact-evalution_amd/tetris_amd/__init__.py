@@ -12,7 +12,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "libtetris_spconv2d.so")
+# TETRIS_SPCONV2D_LIB: another build of the same library (the sanitizer build of `make asan`)
+LIB_PATH = os.environ.get("TETRIS_SPCONV2D_LIB") or os.path.join(os.path.dirname(_HERE), "libtetris_spconv2d.so")
 if not os.path.exists(LIB_PATH):
     raise ImportError("libtetris_spconv2d.so is not built: run `make -C tetris-artifact-evalution_amd` "
                       "(or __graft_entry__.build())")
@@ -46,7 +47,7 @@ BANK_OPTIMIZE = 1
 REORDER_OUT_CHANNEL = 2
 
 OK, EINVAL, EHIP, EUNSUPPORTED, ENOTFOUND, EIO = range(6)
-OPT_PAIRS, OPT_NO_BANK_RULE, OPT_COLD_TIMING = 1, 2, 4  # tetris_options_set
+OPT_PAIRS, OPT_NO_BANK_RULE, OPT_COLD_TIMING, OPT_TRUST_SPF_ARRAYS = 1, 2, 4, 8  # tetris_options_set
 ACT_NONE, ACT_RELU, ACT_RELU_POOL2 = 0, 1, 2  # tetris_spconv2d_launch_act
 
 
@@ -123,7 +124,12 @@ _lib.tetris_noalloc_scratch_limit.restype = C.c_size_t
 _lib.tetris_spconv2d_launch_spf.argtypes = [C.c_void_p] * 7 + [C.c_int] * 8 + [C.c_void_p]
 _lib.tetris_spconv2d_time.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [
     C.POINTER(Tile), C.c_void_p, C.c_int, C.c_int, C.POINTER(C.c_float)]
-_lib.tetris_spconv2d_launch_spf_arrays.argtypes = [C.c_void_p] * 7 + [C.c_int] * 10 + [C.POINTER(Tile), C.c_void_p]
+_lib.tetris_spconv2d_launch_spf_arrays.argtypes = [C.c_void_p] * 7 + [C.c_int] * 10 + [C.c_int64, C.POINTER(Tile),
+                                                                                    C.c_void_p]
+_lib.tetris_spf_invalidate.argtypes = [C.c_void_p]
+_lib.tetris_spf_invalidate.restype = None
+_lib.tetris_spf_check_offsets.argtypes = [np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS"), C.c_int64, C.c_int,
+                                          C.c_int64]
 _lib.tetris_spconv2d_host.argtypes = [_f32p, _f32p, _f32p] + [C.c_int] * 8 + [C.c_void_p, C.c_char_p, C.c_int,
                                                                             C.POINTER(C.c_float)]
 _lib.tetris_spconv2d_spf_host.argtypes = [_f32p, _f32p, _f32p] + [C.c_int] * 8 + [C.c_void_p, C.c_char_p, C.c_int, C.c_uint,
@@ -398,20 +404,33 @@ def tile_autotune_list(filter, batch, img_h, img_w, stride, padding, max_candida
 
 
 def SparseConv2d(input, offsets, stage_len, oc_permutation, position, values, output, batch_size, img_h, img_w,
-                 in_channel, out_channel, kernel_size, stride, padding, stream=0, TILE_IC=0, vec_width=4, tile=None):
+                 in_channel, out_channel, kernel_size, stride, padding, stream=0, TILE_IC=0, vec_width=4, tile=None,
+                 n_entries=0):
     """The reference launcher's call shape on raw device pointers: computes from the arrays passed.  TILE_IC = 0: the
     arrays belong to a live SparseFilter, whose TILE_IC is looked up; else any arrays in that layout
-    (vec_width 4, 1, or 0 for the keep-as-is layout of apply_reorder=False)."""
+    (vec_width 4, 1, or 0 for the keep-as-is layout of apply_reorder=False; n_entries: how many entries `position`
+    and `values` hold, 0 if not known)."""
     if TILE_IC:
         _check(_lib.tetris_spconv2d_launch_spf_arrays(
             C.c_void_p(input), C.c_void_p(offsets), C.c_void_p(stage_len), C.c_void_p(oc_permutation), C.c_void_p(position),
             C.c_void_p(values), C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride,
-            padding, TILE_IC, vec_width, C.byref(tile) if tile is not None else None, C.c_void_p(stream)))
+            padding, TILE_IC, vec_width, n_entries, C.byref(tile) if tile is not None else None, C.c_void_p(stream)))
     else:
         _check(_lib.tetris_spconv2d_launch_spf(C.c_void_p(input), C.c_void_p(offsets), C.c_void_p(stage_len),
                                                C.c_void_p(oc_permutation), C.c_void_p(position), C.c_void_p(values),
                                                C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel,
                                                kernel_size, stride, padding, C.c_void_p(stream)))
+
+
+def spf_invalidate(values):
+    """Forget what the raw launchers remember about the arrays whose values live at device address `values`."""
+    _lib.tetris_spf_invalidate(C.c_void_p(values))
+
+
+def spf_check_offsets(offsets, vec_width, n_entries=0):
+    """The host-side check of a SparseFilter's offsets the raw launchers apply; raises TetrisError(EINVAL)."""
+    o = np.ascontiguousarray(offsets, np.int32)
+    _check(_lib.tetris_spf_check_offsets(o, len(o), vec_width, n_entries))
 
 
 def _host_entry(fn, h_input, h_filter, batch_size, img_h, img_w, in_channel, out_channel, kernel_size, stride, padding,
