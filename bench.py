@@ -93,7 +93,7 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
     if keep and args.save_tiles:
         with open(args.save_tiles, "w") as f:
             json.dump({"suite": suite, "batch": N,
-                       "tiles": [[t.lanes_w, t.quads, t.oc_per_wave, t.waves, t.tile_ic] for t in tiles]}, f)
+                       "tiles": [t.as_list() for t in tiles]}, f)
 
     def step():
         for L, pk, tile, x, y in zip(layers, packs, tiles, xs, ys):
@@ -148,7 +148,7 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
         table.append({"layer": L.name, "us": round(ms * 1e3, 2),
                       "gflops_dense_equiv": round(wk["flops_dense"] / t / 1e9, 1),
                       "bound": wk["bound"], "roofline_frac": round(wk["t_roof"] / t, 4),
-                      "tile": [tile.lanes_w, tile.quads, tile.oc_per_wave, tile.waves, tile.tile_ic]})
+                      "tile": tile.as_list()})
     for pk in packs:
         pk.close()
     fl_dense = sum(w["flops_dense"] for w in works)

@@ -112,6 +112,10 @@ typedef struct tetris_tile {
   int32_t oc_per_wave; /* output channels a wave accumulates at once; oc_per_wave*4*quads <= 128 (64 when waves = 16) */
   int32_t waves;       /* waves per workgroup (1, 2, 4, 8 or 16); it computes waves*oc_per_wave channels */
   int32_t tile_ic;     /* input channels staged in LDS at a time                                   */
+  int32_t csplit;      /* workgroups that share an output tile, each reducing a slice of the input-channel stages
+                          into partial sums that are added afterwards (for layers with too few pixels to fill the
+                          GPU): 1 = none, 2..8 (each slice needs at least two stages), 0 = the library's rule --
+                          split while fewer than half of the GPU's wave slots would be used */
 } tetris_tile;
 
 /* Unmeasured selection: a built-in table of tiles measured on MI355X for the layer shapes of the benchmark
@@ -145,6 +149,16 @@ int tetris_tile_table_load(const char* path, int* rows_out);
  * no read-back, no hash, no synchronisation -- the launch is then as asynchronous as tetris_spconv2d_launch.  A caller
  * that rewrites the arrays in place says so with tetris_spf_invalidate. */
 #define TETRIS_OPT_TRUST_SPF_ARRAYS 8u
+/* Layers whose channel reduction is split over workgroups add their partial sums inside the conv kernel -- the last
+ * wave of every (output tile, wave) pair to finish reads the slices back through L2 and adds them -- instead of in a
+ * second kernel.  Same bits either way.  Measured slower on every suite (the adding wave's loads are a chain of L2
+ * round trips at the end of the kernel, where nothing hides them), so it is a switch for comparing the two, off by
+ * default. */
+#define TETRIS_OPT_ADD_IN_KERNEL 16u
+/* Whether split layers add their slices inside the conv kernel on the current GPU: TETRIS_OPT_ADD_IN_KERNEL is on and
+ * the workgroups whose ids are equal modulo 8 run on one XCD (they then share an L2), which a probe kernel checks once
+ * per device.  No reference counterpart.  Synchronises the device the first time. */
+int tetris_split_layers_add_in_kernel(int* yes);
 int tetris_options_set(unsigned flags);
 unsigned tetris_options_get(void);
 
@@ -230,8 +244,8 @@ int tetris_g950_prepare(tetris_g950* p, int batch, int img_h, int img_w, int str
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  It allocates nothing: the launch plan
  * must exist already (tetris_g950_prepare or an earlier tetris_spconv2d_launch with the same shape and tile, else
  * TETRIS_ENOTFOUND), and the partial sums of a split layer go to a static device array of
- * TETRIS_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends.  A layer whose
- * partial sums need more is refused with TETRIS_EINVAL.  All calls on one GPU share that array: calls that overlap in
+ * TETRIS_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends (64 KiB of it are the
+ * split layers' tickets).  A layer whose partial sums need more is refused with TETRIS_EINVAL.  All calls on one GPU share that array: calls that overlap in
  * time on one GPU (different streams or threads) race; calls on one stream are ordered by the stream.  Results are
  * bit-identical to tetris_spconv2d_launch's. */
 #define TETRIS_NOALLOC_SCRATCH_BYTES (64u << 20)

@@ -24,7 +24,7 @@ def test_bench_line_with_vendor_baselines():
                 "vs_baseline", "dtype", "data", "config", "roofline", "cpu_baseline"):
         assert key in d, key
     assert d["n_gpus"] == 1 and d["steps"] == 3 and d["dtype"] == "f32" and d["vs_baseline"] is None
-    assert d["check"]["ok"] and d["check"]["layers_checked"] == 1
+    assert d["check"]["ok"] and d["check"]["all_workloads_ok"]
     assert d["value"] > 0 and d["ms_per_step"] > 0
     rl = d["roofline"]
     assert rl["bound"] in ("hbm", "mfma") and 0 < rl["frac"] < 1 and rl["peak"] in (8000.0, 157.3)
@@ -32,7 +32,7 @@ def test_bench_line_with_vendor_baselines():
     assert cpu["value"] > 0 and cpu["cores"] >= 1 and cpu["kind"] == "port"
     full = json.load(open(os.path.join(ROOT, d["details"])))  # the side file: per-layer tables and everything else
     assert full["cpu_baseline"]["gpu_vs_this_cpu_output_max_rel_err"] <= 1e-4  # reference-layout decode == device
-    assert len(full["layers"]) == 1 and full["layers"][0]["us"] > 0
+    assert len(full["layers"]) == 1 and full["layers"][0]["us"] > 0 and full["check"]["layers_checked"] == 1
     ctx = d["context"]
     assert ctx["vendor_dense_fp32_ms_per_step"] > 0 and ctx["vendor_csr_im2col_ms_per_step"] > 0, ctx
 

@@ -678,6 +678,72 @@ def test_split_layers_are_bit_reproducible(env):
     pk.close()
 
 
+@pytest.mark.parametrize("case", [
+    # C, K, H, ks, pad, (lanes_w, quads, oc_per_wave, waves, tile_ic)
+    (256, 64, 14, 3, 1, (7, 2, 2, 16, 16)),    # triple-buffered kernel, 16 waves
+    (256, 64, 14, 3, 1, (14, 1, 8, 8, 8)),     # ... 8 waves
+    (128, 32, 7, 3, 1, (7, 1, 8, 4, 8)),       # single-tile kernel
+    (512, 96, 14, 1, 0, (64, 1, 2, 16, 32)),   # flat kernel, 16 waves
+    (512, 96, 7, 1, 0, (64, 2, 4, 8, 16)),     # flat kernel, 8 waves
+])
+def test_slices_of_the_channel_reduction_chosen_by_the_tile(env, case):
+    # tetris_tile.csplit: 1 = none, 2..8 workgroups share an output tile.  Every legal value gives the convolution and
+    # the same bits on a second launch (the slices are added in a fixed order); ReLU on the way out equals ReLU of the
+    # plain result bit for bit; a value that leaves a slice fewer than two stages, or is out of range, is refused.
+    T, torch, O = env
+    C, K, H, ks, pad, t5 = case
+    rng = np.random.default_rng(C + K + H)
+    w = sparse_filter(rng, K, C, ks, 0.85)
+    x = relu_like(rng, (3, C, H, H))
+    ref = O.host_conv2d(x, w, 1, pad, threads=8)
+    stages = -(-C // t5[4])
+    seen = set()
+    for cs in (1, 2, 3, 4, 5, 8):
+        tile = T.Tile(*t5, cs)
+        pk = T.G950Filter.for_tile(w, tile, oc_order="balanced")
+        if stages < 2 * cs:
+            with pytest.raises(T.TetrisError) as e:
+                run_conv(T, torch, pk, x, K, ks, 1, pad, tile)
+            assert e.value.code == T.EINVAL
+            pk.close()
+            continue
+        a = run_conv(T, torch, pk, x, K, ks, 1, pad, tile)
+        b = run_conv(T, torch, pk, x, K, ks, 1, pad, tile)
+        assert not np.isnan(a).any() and a.tobytes() == b.tobytes(), (case, cs)
+        assert max_rel_err(a, ref) <= TOL, (case, cs)
+        # the slices added by the conv kernel's last waves instead of by a second kernel: the same sums in the same order
+        before = T.options_get()
+        try:
+            T.options_set(before | T.OPT_ADD_IN_KERNEL)
+            assert T.split_layers_add_in_kernel()  # MI355X keeps workgroup ids that are equal modulo 8 on one XCD
+            c = run_conv(T, torch, pk, x, K, ks, 1, pad, tile)
+            c2 = run_conv(T, torch, pk, x, K, ks, 1, pad, tile)  # the tickets were left at zero
+        finally:
+            T.options_set(before)
+        assert c2.tobytes() == a.tobytes(), (case, cs)
+        assert c.tobytes() == a.tobytes(), (case, cs)
+        for opts in (before, before | T.OPT_ADD_IN_KERNEL):  # ReLU on the way out, by either adder
+            try:
+                T.options_set(opts)
+                dx = torch.from_numpy(x).cuda()
+                dy = torch.full(ref.shape, float("nan"), device="cuda")
+                pk.launch_act(dx.data_ptr(), dy.data_ptr(), 3, H, H, 1, pad, tile, T.ACT_RELU)
+                torch.cuda.synchronize()
+            finally:
+                T.options_set(before)
+            assert dy.cpu().numpy().tobytes() == np.maximum(a, 0).tobytes(), (case, cs, opts)
+        seen.add(cs)
+        pk.close()
+    assert {1, 2} <= seen
+    assert not T.split_layers_add_in_kernel()  # the switch is off by default
+    pk = T.G950Filter.for_tile(w, T.Tile(*t5), oc_order="balanced")
+    for bad in (9, -1):
+        with pytest.raises(T.TetrisError) as e:
+            run_conv(T, torch, pk, x, K, ks, 1, pad, T.Tile(*t5, bad))
+        assert e.value.code == T.EINVAL
+    pk.close()
+
+
 def test_launches_can_be_captured_in_a_hip_graph(env):
     # After one eager launch per shape (which makes the launch plan and, for a split layer, its scratch buffer) a
     # launch is nothing but kernel launches on the caller's stream, so a chain of layers can be captured once and

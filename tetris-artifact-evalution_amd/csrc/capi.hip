@@ -49,7 +49,7 @@ int find_plan(tetris_g950* p, int N, int H, int W, int stride, int pad, const te
   // a NULL tile is remembered under a key of zeros, so that the library's own choice is made once per shape
   const tetris_tile none{};
   const tetris_tile& kt = given ? *tile : none;
-  const int key[10] = {N, H, W, stride, pad, kt.lanes_w, kt.quads, kt.oc_per_wave, kt.waves, kt.tile_ic};
+  const int key[11] = {N, H, W, stride, pad, kt.lanes_w, kt.quads, kt.oc_per_wave, kt.waves, kt.tile_ic, kt.csplit};
   {
     std::lock_guard<std::mutex> lock(p->mu);
     for (size_t i = p->plans.size(); i-- > 0;)
@@ -88,8 +88,9 @@ int find_plan(tetris_g950* p, int N, int H, int W, int stride, int pad, const te
   return TETRIS_OK;
 }
 
+// scratch of a split layer: the tickets, then csplit copies of the output
 size_t partial_bytes_of(const Geom& g) {
-  return g.csplit > 1 ? sizeof(float) * (size_t)g.csplit * g.N * g.K * g.OH * g.OW : 0;
+  return g.csplit > 1 ? (size_t)kTicketBytes + sizeof(float) * (size_t)g.csplit * g.N * g.K * g.OH * g.OW : 0;
 }
 
 // Partial-sum buffer of a split layer: one per (pack, stream), so that launches of one pack on different streams do
@@ -106,8 +107,17 @@ int partial_buffer(tetris_g950* p, hipStream_t stream, size_t need, bool grow, f
     if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
       return fail(TETRIS_EINVAL, "this launch would allocate its partial-sum buffer: call tetris_g950_prepare before "
                   "capturing");
+    bool same_xcd = false;  // asked here, where allocating and synchronising is allowed, so that launches find the answer
+    int rc = same_xcd_by_residue(&same_xcd);
+    if (rc) return rc;
     float* d = nullptr;
     TETRIS_HIP(hipMalloc(&d, need));
+    // the tickets start at zero; the kernels leave them at zero (this is not under capture: see above)
+    hipError_t e = hipMemsetAsync(d, 0, kTicketBytes, stream);
+    if (e != hipSuccess) {
+      (void)hipFree(d);
+      return fail(TETRIS_EHIP, "clearing the tickets failed: %s", hipGetErrorString(e));
+    }
     if (b.ptr) p->retired.push_back(b.ptr);
     b.ptr = d;
     b.bytes = need;
@@ -132,7 +142,8 @@ int run_launch(tetris_g950* p, const float* d_in, float* d_out, int N, int H, in
 }
 
 // ---- scratch of the entry point that allocates nothing ------------------------------------------------------------
-// Partial sums of split layers for callers that cannot allocate.  One array per GPU, held until the process ends;
+// Tickets and partial sums of split layers for callers that cannot allocate.  One array per GPU, held until the
+// process ends (zero when the code object is loaded: the tickets start at zero, and every launch leaves them so);
 // every call on a GPU shares it, so calls that overlap in time on one GPU race.
 constexpr size_t kStaticScratchBytes = (size_t)TETRIS_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) __attribute__((used)) float scratch[kStaticScratchBytes / sizeof(float)];
@@ -151,6 +162,9 @@ int static_scratch(float** out) {
     void* ptr = nullptr;
     TETRIS_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
     if (!ptr) return fail(TETRIS_EHIP, "hipGetSymbolAddress returned a null address for the scratch array");
+    bool same_xcd = false;  // the placement probe of split layers, made here so that launches find the answer ready
+    const int rc = same_xcd_by_residue(&same_xcd);
+    if (rc) return rc;
     g_scratch_ptr[dev] = static_cast<float*>(ptr);
   }
   *out = g_scratch_ptr[dev];
@@ -568,7 +582,8 @@ int tetris_spf_device_arrays(tetris_spf* f, tetris_spf_arrays* o) {
 }
 
 int tetris_options_set(unsigned flags) {
-  if (flags & ~(TETRIS_OPT_PAIRS | TETRIS_OPT_NO_BANK_RULE | TETRIS_OPT_COLD_TIMING | TETRIS_OPT_TRUST_SPF_ARRAYS))
+  if (flags & ~(TETRIS_OPT_PAIRS | TETRIS_OPT_NO_BANK_RULE | TETRIS_OPT_COLD_TIMING | TETRIS_OPT_TRUST_SPF_ARRAYS |
+                TETRIS_OPT_ADD_IN_KERNEL))
     return fail(TETRIS_EINVAL, "unknown option bits 0x%x", flags);
   set_options(flags);
   return TETRIS_OK;
@@ -651,8 +666,37 @@ int tetris_tile_autotune_list(const float* h_filter, int N, int H, int W, int C,
     timed.emplace_back(ms, t);
   }
   if (timed.empty()) return done(fail(TETRIS_EINVAL, "no tile shape could be launched for this layer"));
-  std::stable_sort(timed.begin(), timed.end(),
-                   [](const std::pair<float, tetris_tile>& a, const std::pair<float, tetris_tile>& b) { return a.first < b.first; });
+  auto by_time = [](const std::pair<float, tetris_tile>& a, const std::pair<float, tetris_tile>& b) { return a.first < b.first; };
+  std::stable_sort(timed.begin(), timed.end(), by_time);
+  // The candidates so far leave the split of the channel reduction to the rule.  For the fastest of them, where the
+  // layer has few enough pixels for a split to be legal, time the other slice counts too (1 = none, 2, 4, 8): fewer
+  // slices move fewer partial sums, more slices fill more of the GPU.
+  {
+    const size_t top = std::min<size_t>(timed.size(), 6);
+    std::vector<std::pair<float, tetris_tile>> extra;
+    for (size_t i = 0; i < top; ++i) {
+      const tetris_tile base = timed[i].second;
+      tetris_g950* pk = packs[{base.tile_ic, base.oc_per_wave, base.waves}];
+      Geom g0;
+      if (make_geom(pk, N, H, W, stride, pad, base, &g0) != TETRIS_OK) continue;
+      for (int cs : {1, 2, 4, 8}) {
+        if (cs == g0.csplit) continue;
+        tetris_tile v = base;
+        v.csplit = cs;
+        Geom gv;
+        if (make_geom(pk, N, H, W, stride, pad, v, &gv) != TETRIS_OK) continue;
+        // more slices than wave slots to run them at once only add partial sums
+        if (cs > g0.csplit && (long long)gv.ugroups * gv.kblocks * cs * v.waves > 16ll * 256 * 2) continue;
+        float ms = 0;
+        rc = time_launches(pk, d_in, d_out, N, H, W, stride, pad, &v, stream, 1, 3, &ms);
+        if (rc == TETRIS_EINVAL) continue;
+        if (rc) return done(rc);
+        extra.emplace_back(ms, v);
+      }
+    }
+    timed.insert(timed.end(), extra.begin(), extra.end());
+    std::stable_sort(timed.begin(), timed.end(), by_time);
+  }
   const size_t again = std::min<size_t>(timed.size(), std::max(4, max_out));
   for (size_t i = 0; i < again; ++i) {
     const tetris_tile& t = timed[i].second;
@@ -662,8 +706,7 @@ int tetris_tile_autotune_list(const float* h_filter, int N, int H, int W, int C,
     if (rc) return done(rc);
     timed[i].first = ms;
   }
-  std::stable_sort(timed.begin(), timed.begin() + again,
-                   [](const std::pair<float, tetris_tile>& a, const std::pair<float, tetris_tile>& b) { return a.first < b.first; });
+  std::stable_sort(timed.begin(), timed.begin() + again, by_time);
   const int n = (int)std::min<size_t>(again, (size_t)max_out);
   for (int i = 0; i < n; ++i) {
     out[i] = timed[i].second;
@@ -719,6 +762,15 @@ int tetris_g950_prepare(tetris_g950* p, int N, int H, int W, int stride, int pad
   return static_scratch(&s);  // looks the static scratch array of this GPU up, for tetris_spconv2d_launch_noalloc
 }
 
+int tetris_split_layers_add_in_kernel(int* yes) {
+  if (!yes) return fail(TETRIS_EINVAL, "null argument");
+  bool ok = false;
+  const int rc = same_xcd_by_residue(&ok);
+  if (rc) return rc;
+  *yes = ok && (options() & TETRIS_OPT_ADD_IN_KERNEL);
+  return TETRIS_OK;
+}
+
 size_t tetris_noalloc_scratch_bytes(void) { return g_scratch_limit.load(); }
 
 size_t tetris_noalloc_scratch_limit(size_t bytes) {
@@ -739,8 +791,8 @@ int tetris_spconv2d_launch_noalloc(tetris_g950* p, const float* d_in, float* d_o
     const size_t need = partial_bytes_of(plan.geom);
     const size_t limit = g_scratch_limit.load();
     if (need > limit)
-      return fail(TETRIS_EINVAL, "this layer needs %zu bytes of partial sums, the static scratch holds %zu: use "
-                  "tetris_spconv2d_launch", need, limit);
+      return fail(TETRIS_EINVAL, "this layer needs %zu bytes of tickets and partial sums, the static scratch holds %zu: "
+                  "use tetris_spconv2d_launch", need, limit);
     rc = static_scratch(&d_partial);
     if (rc) return rc;
   }

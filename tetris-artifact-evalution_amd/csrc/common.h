@@ -45,6 +45,10 @@ constexpr int kAccRegs = 128;    // accumulator VGPRs of a wave: oc_per_wave * 4
 constexpr int kFillItems = 8;    // staged 16-byte slots a thread may hold in flight per stage
 constexpr int kFlatLanes = 64;   // tetris_tile.lanes_w of the flat (pointwise) tiles
 constexpr int kMaxSplit = 8;      // most workgroups that may share an output tile (each reduces a slice of the stages)
+// A split layer's scratch starts with its tickets -- one int per (output tile, wave), zero between launches -- and
+// the partial sums follow.
+constexpr int kTicketBytes = 65536;
+constexpr int kMaxTickets = kTicketBytes / 4;
 
 inline int out_extent(int in, int pad, int ks, int stride) { return (in + 2 * pad - ks) / stride + 1; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -123,6 +127,10 @@ struct Geom {
   // What a kernel does to a finished sum before it writes it (set per launch): 0 nothing, 1 ReLU, 2 ReLU and 2x2
   // max-pooling inside the halo'd kernels (the output tensor is then N x K x OH/2 x OW/2).
   int act;
+  // Split layers (csplit > 1), set per launch: 1 = every wave, once its partial sums are stored, takes a ticket of its
+  // (output tile, wave) pair, and the wave that draws the last one adds the slices itself, in slice order, and writes
+  // the finished sums (through `act` 0 or 1); 0 = a second kernel adds the slices.
+  int fused;
   // multiply-high reciprocals, floor(2^32 / d) + 1: x / d == umulhi(x, m) whenever x * d < 2^32
   unsigned m_per_unit, m_cpp, m_pitch, m_par, m_upi, m_units_w, m_lr, m_thi, m_kblocks, m_csplit;
   unsigned m_fill_slots, m_slots_per_unit, m_per_img, m_per_row, m_ng;  // single-tile kernel's staging plan
@@ -154,7 +162,7 @@ struct BoundKey {
 namespace tetris {
 // A launch plan: everything run_launch derives from (input shape, tile) for one pack, kept for the next call.
 struct Plan {
-  int key[10];  // N, H, W, stride, pad, lanes_w, quads, oc_per_wave, waves, tile_ic
+  int key[11];  // N, H, W, stride, pad, lanes_w, quads, oc_per_wave, waves, tile_ic, csplit
   Geom geom;
   const int2* entries;        // the pack's entries bound to the geometry
   const int32_t* grp_off;     // [groups*stages+1] first entry of every stream in `entries`
@@ -251,12 +259,18 @@ int balance_oc_order(const float* filter, int C, int K, int ks, const tetris_til
 
 // spconv2d_kernel.hip
 // launches the conv; when the geometry splits the channel reduction (csplit > 1) the workgroups write their partial
-// sums to d_partial ([csplit] outputs) and a second kernel adds the slices, in order, into d_out
+// sums to the scratch ([csplit] outputs) and the slices are added, in slice order, into d_out: by the last wave of
+// every (tile, wave) pair to finish (TETRIS_OPT_ADD_IN_KERNEL, on a device whose workgroup placement keeps a tile's
+// slices on one XCD, no pooling), or else by a second kernel
 // act: 0 = d_out gets the sums; 1 = their ReLU; 2 = ReLU and 2x2 max-pooling (d_out is N x K x OH/2 x OW/2), done by
 // the adding kernel of a split layer and otherwise inside the conv kernel where geom_pools_in_kernel allows (else
 // TETRIS_EUNSUPPORTED, nothing launched)
-int launch_conv(const Geom& g, const float* d_in, float* d_out, float* d_partial, const int2* entries,
+// d_scratch (split layers): kTicketBytes of tickets, all zero between launches, then room for csplit outputs
+int launch_conv(const Geom& g, const float* d_in, float* d_out, float* d_scratch, const int2* entries,
                 const int32_t* grp_off, const int32_t* grp_pair, const int32_t* oc_order, int act, hipStream_t stream);
+// whether workgroups with the same blockIdx.x % 8 run on one XCD of the current device (probed once per device):
+// what lets the slices of a split layer exchange their partial sums through that XCD's L2
+int same_xcd_by_residue(bool* ok);
 bool geom_pools_in_kernel(const Geom& g);
 // whether the kernel of geometry `g` walks paired streams
 bool geom_walks_pairs(const Geom& g);

@@ -104,6 +104,20 @@ int image_stride(const Shape& s, int tile_ic, int stride) {
 
 }  // namespace
 
+// How many workgroups share an output tile.  The tile may say (1 = none, up to kMaxSplit, every slice at least two
+// stages); 0 leaves it to the rule: small feature maps leave most of the CUs without a workgroup, so double the
+// slices while fewer than half of the wave slots (`room`) would be used and every slice keeps at least four stages.
+static int choose_csplit(const tetris_tile& t, long long waves_total, long long room, int stages, int* out) {
+  if (t.csplit < 0 || t.csplit > kMaxSplit) return fail(TETRIS_EINVAL, "bad tile: csplit=%d (0..%d)", t.csplit, kMaxSplit);
+  if (t.csplit > 1 && stages < 2 * t.csplit)
+    return fail(TETRIS_EINVAL, "bad tile: %d slices of %d stages (every slice needs at least two)", t.csplit, stages);
+  int cs = 1;
+  if (t.csplit > 0) cs = t.csplit;
+  else while (cs < kMaxSplit && waves_total * cs * 2 <= room && stages >= 8 * cs) cs *= 2;
+  *out = cs;
+  return TETRIS_OK;
+}
+
 // Geometry of a flat tile (lanes_w == 64) for a pointwise layer; `g` holds the layer and the tile's quads, slots and waves.
 static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Geom* out) {
   if (p->ks != 1 || g.stride != 1 || g.pad != 0 || g.step < 1)  // a strided layer arrives as stride 1 on its sub-grid
@@ -148,11 +162,12 @@ static int make_flat_geom(const tetris_g950* p, Geom g, const tetris_tile& t, Ge
   const bool four = t.waves == 16 || g.buf_bytes == kFlatHalfBufBytes;
   const long long room = (long long)cu_count() * (four ? 16 : 8);
   const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
-  g.csplit = 1;
-  while (g.csplit < kMaxSplit && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
+  if (int rc = choose_csplit(t, waves_total, room, g.stages, &g.csplit)) return rc;
   if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32) ||
       (long long)g.stages * (g.csplit + 1) * g.csplit >= (1ll << 32))
     return fail(TETRIS_EINVAL, "grid too large");
+  if (g.csplit > 1 && 4ll * g.csplit * g.N * p->K * hw > (1ll << 30))
+    return fail(TETRIS_EINVAL, "%d slices of this layer's output are more than 1 GiB of partial sums", g.csplit);
   g.m_kblocks = magic_reciprocal(g.kblocks);
   g.m_csplit = magic_reciprocal(g.csplit);
   g.stagers = t.waves;
@@ -244,10 +259,11 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     const bool four = t.waves == 16 || g.buf_bytes == kHalfBufBytes;  // waves per SIMD the kernel variant allows
     const long long room = (long long)cu_count() * (g.ver == 3 && four ? 16 : 8);
     const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
-    g.csplit = 1;
-    while (g.csplit < kMaxSplit && waves_total * g.csplit * 2 <= room && g.stages >= 8 * g.csplit) g.csplit *= 2;
+    if (int rc = choose_csplit(t, waves_total, room, g.stages, &g.csplit)) return rc;
     if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32))
       return fail(TETRIS_EINVAL, "grid too large");
+    if (g.csplit > 1 && 4ll * g.csplit * N * p->K * g.OH * g.OW > (1ll << 30))
+      return fail(TETRIS_EINVAL, "%d slices of this layer's output are more than 1 GiB of partial sums", g.csplit);
     g.m_kblocks = magic_reciprocal(g.kblocks);
     g.m_csplit = magic_reciprocal(g.csplit);
   }
@@ -435,7 +451,7 @@ struct Tuned {
 };
 const Tuned kTuned[] = {
 #include "tuned_tiles.inc"
-    {0, 0, 0, 0, 0, 0, 0, 0, {0, 0, 0, 0, 0}}};
+    {0, 0, 0, 0, 0, 0, 0, 0, {0, 0, 0, 0, 0, 0}}};
 
 // Rows a caller loaded at run time (tetris_tile_table_load); they are looked up before the built-in ones.
 std::mutex g_loaded_mu;
@@ -463,11 +479,13 @@ int load_tile_table(const char* path, int* rows_out) {
   std::vector<Tuned> rows;
   char line[512];
   while (std::fgets(line, sizeof line, fp)) {
-    Tuned e;
-    if (std::sscanf(line, " {%d, %d, %d, %d, %d, %d, %d, %d, {%d, %d, %d, %d, %d}}", &e.N, &e.H, &e.W, &e.C, &e.K, &e.ks,
-                    &e.stride, &e.pad, &e.tile.lanes_w, &e.tile.quads, &e.tile.oc_per_wave, &e.tile.waves,
-                    &e.tile.tile_ic) == 13)
-      rows.push_back(e);
+    Tuned e{};
+    // the tile's sixth number (csplit) is optional: a row without it leaves the split to the library's rule
+    const int n = std::sscanf(line, " {%d, %d, %d, %d, %d, %d, %d, %d, {%d, %d, %d, %d, %d, %d}}", &e.N, &e.H, &e.W, &e.C, &e.K,
+                              &e.ks, &e.stride, &e.pad, &e.tile.lanes_w, &e.tile.quads, &e.tile.oc_per_wave, &e.tile.waves,
+                              &e.tile.tile_ic, &e.tile.csplit);
+    if (n == 13) e.tile.csplit = 0;
+    if (n >= 13) rows.push_back(e);
   }
   std::fclose(fp);
   std::lock_guard<std::mutex> lock(g_loaded_mu);

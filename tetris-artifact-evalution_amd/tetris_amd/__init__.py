@@ -47,7 +47,7 @@ BANK_OPTIMIZE = 1
 REORDER_OUT_CHANNEL = 2
 
 OK, EINVAL, EHIP, EUNSUPPORTED, ENOTFOUND, EIO = range(6)
-OPT_PAIRS, OPT_NO_BANK_RULE, OPT_COLD_TIMING, OPT_TRUST_SPF_ARRAYS = 1, 2, 4, 8  # tetris_options_set
+OPT_PAIRS, OPT_NO_BANK_RULE, OPT_COLD_TIMING, OPT_TRUST_SPF_ARRAYS, OPT_ADD_IN_KERNEL = 1, 2, 4, 8, 16  # tetris_options_set
 ACT_NONE, ACT_RELU, ACT_RELU_POOL2 = 0, 1, 2  # tetris_spconv2d_launch_act
 
 
@@ -72,13 +72,20 @@ class _G950Arrays(C.Structure):
 
 
 class Tile(C.Structure):
-    """tetris_tile: lanes_w, quads, oc_per_wave, waves, tile_ic (all zero = let the library choose)."""
+    """tetris_tile: lanes_w, quads, oc_per_wave, waves, tile_ic (all zero = let the library choose) and csplit
+    (slices of the channel reduction: 0 = the library's rule, 1 = none, 2..8)."""
     _fields_ = [("lanes_w", C.c_int32), ("quads", C.c_int32), ("oc_per_wave", C.c_int32), ("waves", C.c_int32),
-                ("tile_ic", C.c_int32)]
+                ("tile_ic", C.c_int32), ("csplit", C.c_int32)]
+
+    def as_list(self):
+        """[lanes_w, quads, oc_per_wave, waves, tile_ic], plus csplit when the tile fixes it."""
+        five = [self.lanes_w, self.quads, self.oc_per_wave, self.waves, self.tile_ic]
+        return five + [self.csplit] if self.csplit else five
 
     def __repr__(self):
-        return "Tile(lanes_w=%d, quads=%d, oc_per_wave=%d, waves=%d, tile_ic=%d)" % (
-            self.lanes_w, self.quads, self.oc_per_wave, self.waves, self.tile_ic)
+        return "Tile(lanes_w=%d, quads=%d, oc_per_wave=%d, waves=%d, tile_ic=%d%s)" % (
+            self.lanes_w, self.quads, self.oc_per_wave, self.waves, self.tile_ic,
+            ", csplit=%d" % self.csplit if self.csplit else "")
 
 
 _f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
@@ -399,7 +406,8 @@ def tile_autotune_list(filter, batch, img_h, img_w, stride, padding, max_candida
     tiles, ms, n = (Tile * max_out)(), (C.c_float * max_out)(), C.c_int()
     _check(_lib.tetris_tile_autotune_list(w, batch, img_h, img_w, Cc, K, ks, stride, padding, max_candidates,
                                           C.c_void_p(stream), tiles, ms, max_out, C.byref(n)))
-    return [(Tile(tiles[i].lanes_w, tiles[i].quads, tiles[i].oc_per_wave, tiles[i].waves, tiles[i].tile_ic), float(ms[i]))
+    return [(Tile(tiles[i].lanes_w, tiles[i].quads, tiles[i].oc_per_wave, tiles[i].waves, tiles[i].tile_ic,
+                  tiles[i].csplit), float(ms[i]))
             for i in range(n.value)]
 
 
@@ -420,6 +428,13 @@ def SparseConv2d(input, offsets, stage_len, oc_permutation, position, values, ou
                                                C.c_void_p(oc_permutation), C.c_void_p(position), C.c_void_p(values),
                                                C.c_void_p(output), batch_size, img_h, img_w, in_channel, out_channel,
                                                kernel_size, stride, padding, C.c_void_p(stream)))
+
+
+def split_layers_add_in_kernel():
+    """Whether layers whose channel reduction is split add their slices inside the conv kernel on this GPU."""
+    yes = C.c_int(0)
+    _check(_lib.tetris_split_layers_add_in_kernel(C.byref(yes)))
+    return bool(yes.value)
 
 
 def spf_invalidate(values):
