@@ -224,6 +224,23 @@ int tetris_spconv2d_launch(tetris_g950* p, const float* d_input, float* d_output
  * in *supported; launch with TETRIS_ACT_RELU and pool with tetris_relu_maxpool then).  Results are
  * bit-identical to tetris_spconv2d_launch followed by tetris_relu_maxpool.  Plans, scratch and graph capture as for
  * tetris_spconv2d_launch. */
+/* How a layer is cut into workgroups for a tile, without launching anything: what the launcher derives from
+ * (input shape, tile) before it launches.  No reference counterpart (the reference's grid follows from its template
+ * arguments, Tetris/spconv2d_kernel.cu:163-188). */
+typedef struct tetris_launch_shape {
+  int32_t workgroups;     /* unit_groups * channel_blocks * csplit */
+  int32_t unit_groups;    /* workgroups along the output pixels (each `quads` units of up to 256 pixels) */
+  int32_t channel_blocks; /* workgroups along the output channels (each waves * oc_per_wave channels) */
+  int32_t csplit;         /* workgroups that share an output tile (the tile's value, or the rule's when that is 0) */
+  int32_t stages;         /* input-channel stages of the whole reduction: ceil(in_channel / tile_ic) */
+  int32_t lanes_used;     /* lanes of a wave that own pixels, out of 64 */
+  int32_t kernel;         /* 2 single LDS tile, 3 three LDS buffers, 4 flat tile of pointwise layers */
+  int32_t lds_bytes;      /* dynamic LDS of a workgroup */
+  int64_t scratch_bytes;  /* tickets + partial sums a split layer needs (0 when csplit is 1) */
+} tetris_launch_shape;
+int tetris_launch_shape_of(tetris_g950* p, int batch, int img_h, int img_w, int stride, int padding,
+                           const tetris_tile* tile, tetris_launch_shape* out);
+
 #define TETRIS_ACT_NONE 0
 #define TETRIS_ACT_RELU 1
 #define TETRIS_ACT_RELU_POOL2 2

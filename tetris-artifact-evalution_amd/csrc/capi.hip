@@ -747,6 +747,24 @@ int tetris_spconv2d_act_supported(tetris_g950* p, int N, int H, int W, int strid
   return TETRIS_OK;
 }
 
+int tetris_launch_shape_of(tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile* tile,
+                           tetris_launch_shape* out) {
+  if (!p || !tile || !out) return fail(TETRIS_EINVAL, "null argument");
+  Geom g;
+  const int rc = make_geom(p, N, H, W, stride, pad, *tile, &g);
+  if (rc) return rc;
+  out->unit_groups = g.ugroups;
+  out->channel_blocks = g.kblocks;
+  out->csplit = g.csplit;
+  out->workgroups = g.ugroups * g.kblocks * g.csplit;
+  out->stages = g.stages;
+  out->lanes_used = g.ver == 4 ? 64 : g.lw * std::min(g.lh, g.thi * g.nb);
+  out->kernel = g.ver;
+  out->lds_bytes = g.ver == 4 ? 2 * g.buf_bytes : g.ver == 3 ? kBufs * g.buf_bytes : kTileBytes;
+  out->scratch_bytes = (int64_t)partial_bytes_of(g);
+  return TETRIS_OK;
+}
+
 int tetris_g950_prepare(tetris_g950* p, int N, int H, int W, int stride, int pad, const tetris_tile* tile, void* stream_) {
   if (!p) return fail(TETRIS_EINVAL, "null argument");
   hipStream_t stream = static_cast<hipStream_t>(stream_);

@@ -50,6 +50,52 @@ __device__ __forceinline__ void touch_kernel_arguments() {
   asm volatile("" ::"s"(a0), "s"(a1), "s"(a2), "s"(a3), "s"(a4), "s"(a5));
 }
 
+// Time stamps of a workgroup's life, compiled in by -DTETRIS_STAMPS only (`make stamps`; read with tetris_stamps_read,
+// printed by `python -m tetris_amd.stamps`).  Wave 0 of workgroup `logical` records the shader clock where the kernels
+// say TETRIS_STAMP(i): 0 kernel entry, 1 kernel arguments touched, 2 first stage's input loads issued, 3 stream offsets
+// and first batch in scalar registers, 4 first stage landed and barrier passed, 5 stage loop left, 6 output stores
+// issued, 7 output stores acknowledged, 11 staging plan made (just before the first loads go out); slot 8 adds up the
+// clocks wave 0 spent inside the walk (12: the largest such sum over the workgroup's waves, 13: the sum over its
+// waves), 9 and 10 hold the 100 MHz wall clock at entry and at the end (the clocks' ratio, and when the workgroup ran
+// within the launch).
+#ifdef TETRIS_STAMPS
+constexpr int kStampSlots = 16, kStampWgs = 8192;
+__device__ long long g_stamps[kStampWgs * kStampSlots];
+#define TETRIS_STAMP_ENTRY() const long long stamp_t0_ = clock64(), stamp_w0_ = wall_clock64(); long long stamp_t1_ = 0, stamp_walk_ = 0
+#define TETRIS_STAMP_ARGS() stamp_t1_ = clock64()
+#define TETRIS_STAMP(i)                                                                                           \
+  do {                                                                                                            \
+    if (threadIdx.x == 0 && logical < kStampWgs) g_stamps[logical * kStampSlots + (i)] = clock64();                \
+  } while (0)
+#define TETRIS_STAMP_WALK(statement)                                                                              \
+  do {                                                                                                            \
+    const long long w0_ = clock64();                                                                              \
+    statement;                                                                                                    \
+    stamp_walk_ += clock64() - w0_;                                                                               \
+  } while (0)
+#define TETRIS_STAMP_END()                                                                                        \
+  do {                                                                                                            \
+    TETRIS_STAMP(6);                                                                                              \
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                                              \
+    if ((threadIdx.x & 63) == 0 && logical < kStampWgs) {  /* every wave: the busiest wave's walk and the sum */    \
+      unsigned long long* u_ = reinterpret_cast<unsigned long long*>(g_stamps + logical * kStampSlots);           \
+      atomicMax(u_ + 12, (unsigned long long)stamp_walk_);                                                        \
+      atomicAdd(u_ + 13, (unsigned long long)stamp_walk_);                                                        \
+    }                                                                                                             \
+    if (threadIdx.x == 0 && logical < kStampWgs) {                                                                \
+      long long* s_ = g_stamps + logical * kStampSlots;                                                           \
+      s_[0] = stamp_t0_; s_[1] = stamp_t1_; s_[7] = clock64(); s_[8] = stamp_walk_; s_[9] = stamp_w0_;            \
+      s_[10] = wall_clock64();                                                                                    \
+    }                                                                                                             \
+  } while (0)
+#else
+#define TETRIS_STAMP_ENTRY() do {} while (0)
+#define TETRIS_STAMP_ARGS() do {} while (0)
+#define TETRIS_STAMP(i) do {} while (0)
+#define TETRIS_STAMP_WALK(statement) statement
+#define TETRIS_STAMP_END() do {} while (0)
+#endif
+
 // s36..s51 (the current batch) and s72:s73 (the stream address) are operands of the walk, bound by their constraints
 #define TETRIS_S_CLOBBERS                                                                                          \
   "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68",   \
@@ -394,7 +440,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(88))) void spco
     const int32_t* __restrict__ grp_off, const int32_t* __restrict__ grp_pair,
     const int32_t* __restrict__ oc_order, float* __restrict__ final_out, int* __restrict__ tickets, const Geom g) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  TETRIS_STAMP_ENTRY();
   touch_kernel_arguments();
+  TETRIS_STAMP_ARGS();
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = uniform(tid >> 6);
@@ -412,7 +460,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(88))) void spco
   const int ugroup = fast_div(tile_id, g.m_kblocks);
   const int kblock = tile_id - ugroup * g.kblocks;
   const int u0 = ugroup * NQ;
-  const int st0 = slice * g.stages / g.csplit, st1 = (slice + 1) * g.stages / g.csplit;  // this workgroup's stages
+  // this workgroup's stages (multiply-high division: make_geom checks its range)
+  const int st0 = fast_div(slice * g.stages, g.m_csplit), st1 = fast_div((slice + 1) * g.stages, g.m_csplit);
   // a slice of a split reduction writes its partial sums to its own copy of the output (`out` is then that scratch)
   const size_t out_elems = (size_t)g.N * g.K * g.OH * g.OW;
   const int upi = g.units_w * g.units_h;  // units per image block
@@ -526,6 +575,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(88))) void spco
   const int2* stream = entries + o0 + 8;
   Batch head;
   spread_head(head, head_entry);
+  TETRIS_STAMP(3);
 
   // The scalar loads of the walk run only one 64-byte fetch ahead, far too little to cover a miss in L2.  So each
   // wave touches the stream of the stage after next with one vector load (a dword per 128-byte line, 8 KB at most)
@@ -538,21 +588,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(88))) void spco
   int sink = touch(o0 + 8, o_end);  // as much of the wave's whole stream as one touch covers (8 KB)
   int touched = 0;
 
+  TETRIS_STAMP(11);
   fetch(st0);
+  TETRIS_STAMP(2);
   for (int st = st0; st < st1; ++st) {
     commit();
     sink ^= touched;
     __syncthreads();
+    if (st == st0) TETRIS_STAMP(4);
     if (st + 1 < st1) fetch(st + 1);  // in flight while this stage is computed
     const int o3 = uniform(go[min(st + 3, g.stages)]);  // stream bounds two stages ahead
     touched = touch(o2, o3);
     const int nb = (o1 - o0) >> 3;
     const int np = uniform(gp[st]) >> 3;  // the stream's batches of pairs come first
-    if (np > 0) walk_stream<NQ, 2, 2>(head, stream, np, lane_base, (wave >> 2) * 2 + st);
-    if (nb - np > 0) walk_stream<NQ, 2, 1>(head, stream, nb - np, lane_base, (wave >> 2) * 2 + st + 1);
+    if (np > 0) TETRIS_STAMP_WALK((walk_stream<NQ, 2, 2>(head, stream, np, lane_base, (wave >> 2) * 2 + st)));
+    if (nb - np > 0) TETRIS_STAMP_WALK((walk_stream<NQ, 2, 1>(head, stream, nb - np, lane_base, (wave >> 2) * 2 + st + 1)));
     o0 = o1; o1 = o2; o2 = o3;
     __syncthreads();  // everyone is done reading the tile
   }
+  TETRIS_STAMP(5);
 
   // ---- write the outputs -------------------------------------------------------------------------------------
   if (g.N < 0) out[0] = __builtin_bit_cast(float, sink ^ touched);  // never true: keeps the touching loads alive
@@ -560,6 +614,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_num_vgpr(88))) void spco
   else store_outputs<NQ, 2>(out + (size_t)slice * out_elems, lane_oc, g, u0, n_base, limg, lrow, lx, lane_ok);
   if (g.fused && drew_last_ticket(tickets, tile_id, wave, g))
     add_slices<NQ>(out, final_out, lane_oc, g, u0, n_base, limg, lrow, lx, lane_ok);
+  TETRIS_STAMP_END();
 }
 
 static_assert(TETRIS_WALK_TILE_BYTES == kTileBytes && TETRIS_WALK_BUF_BYTES == kBufBytes &&
@@ -586,7 +641,9 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
   constexpr int MAXC = VARIANT == 3 ? kMaxChunks : kMaxChunks16;
   constexpr int BUF = VARIANT == 5 ? kHalfBufBytes : kBufBytes;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  TETRIS_STAMP_ENTRY();
   touch_kernel_arguments();
+  TETRIS_STAMP_ARGS();
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = uniform(tid >> 6);
@@ -600,13 +657,12 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
   const int ugroup = fast_div(tile_id, g.m_kblocks);
   const int kblock = tile_id - ugroup * g.kblocks;
   const int u0 = ugroup * NQ;
-  const int st0 = slice * g.stages / g.csplit, st1 = (slice + 1) * g.stages / g.csplit;  // this workgroup's stages
+  // this workgroup's stages (multiply-high division: make_geom checks its range)
+  const int st0 = fast_div(slice * g.stages, g.m_csplit), st1 = fast_div((slice + 1) * g.stages, g.m_csplit);
   // a slice of a split reduction writes its partial sums to its own copy of the output (`out` is then that scratch)
   const size_t out_elems = (size_t)g.N * g.K * g.OH * g.OW;
   const int upi = g.units_w * g.units_h;
   const int n_base = fast_div(u0, g.m_upi) * g.nb * g.fold;
-
-  zero_accumulators<VARIANT>(g.g * 4 * NQ);
 
   const size_t hw = (size_t)g.in_hw;  // floats per (image, channel) plane in memory
   const float* in_base = in + (size_t)n_base * g.C * hw;
@@ -623,10 +679,17 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
   bool writes[MAXC];     // this lane's dword lies inside the plane (the last chunk of a plane may overhang)
   // chunks this wave stages: x = wave, wave + stagers, ... below nchunks -- a wave-uniform count, so that the plan
   // and every issue() skip the other slots with scalar branches (a load under an empty exec mask still costs its issue)
+  TETRIS_STAMP(11);
   const int stager_shift = g.stagers == 16 ? 4 : g.stagers == 8 ? 3 : 2;  // stagers is 4, 8 or 16
   const int n_live = wave < g.stagers ? min(g.ni, (g.nchunks - wave + g.stagers - 1) >> stager_shift) : 0;
+  // The plan of a chunk costs some hundred cycles of index arithmetic, and the loads of a stage keep the CU's address
+  // unit busy for about as long as the whole plan takes: so the first stage's loads of chunk i go out as soon as chunk
+  // i's plan is made, and the address unit works while the plan of chunk i + 1 is computed.
   {
     const int per_unit = g.nb * g.cpp;
+    unsigned char* buf0 = smem + (st0 % kBufs) * BUF;
+    const int c00 = st0 * g.tile_ic;
+    const int nch0 = min(g.tile_ic, g.C - c00);
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
       writes[i] = false;
@@ -657,6 +720,11 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
                       col < g.W;
       voff[i] = ok ? (unsigned)(((n - n_base) * g.C) * (int)hw + ihh * g.step * g.in_w + col * g.step) * 4u : kInvalid;
       loff[i] = uniform(q * g.region + 4 * (img * g.img_stride + chunk * 64));
+      if (writes[i])
+        for (int ch = 0; ch < nch0; ++ch)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(
+              rsrc, (__attribute__((address_space(3))) void*)(buf0 + loff[i] + 4 * ch * g.plane), 4, (int)voff[i],
+              (c00 + ch) * (int)hw * 4, 0, 0);
     }
   }
   auto issue = [&](int st) {  // start the loads of stage `st` into buffer st % 3
@@ -685,10 +753,11 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
   // stage st0 + 1 are issued then and land during the first half of the walk (-1 % per launch).  When everybody
   // stages it pays to have both stages in flight before the first wait (measured both ways).
   const bool early_start = WAVES == 16 || !split;
-  // The first stage's loads go out before anything else is fetched (the streams' offsets and head entries, the
-  // wave's channels), so that those round trips run under the input's.
-  issue(st0);
+  // The first stage's loads have gone out (with the plan, above) before anything else is fetched (the streams'
+  // offsets and head entries, the wave's channels), so that those round trips run under the input's.
   if (!early_start) issue(st0 + 1);
+  TETRIS_STAMP(2);
+  zero_accumulators<VARIANT>(g.g * 4 * NQ);
 
   // ---- lane -> pixels -------------------------------------------------------------------------------------------
   const int ly = fast_div(lane, g.m_lr);
@@ -712,6 +781,7 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
   const int2* stream = entries + o0 + 8;
   Batch head;
   spread_head(head, head_entry);
+  TETRIS_STAMP(3);
 
   const int* words = reinterpret_cast<const int*>(entries);
   auto touch = [&](int from, int to) {  // pull a stream range into L2: a dword per 128-byte line, 8 KB at most
@@ -722,6 +792,7 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
 
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0); the expcnt and lgkmcnt fields stay at their maxima
   __syncthreads();
+  TETRIS_STAMP(4);
   if (early_start) issue(st0 + 1);
   for (int st = st0; st < st1; ++st) {
     const int o4 = uniform(go[min(st + 4, g.stages)]);  // fetched an iteration before it is needed
@@ -735,16 +806,18 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
     // result carried into the next iteration may be given a register copy at the loop's end, and that copy waits for
     // every load in flight, the next stage's included.
     const int touched = touch(o2, o3);
-    if (np > 0) walk_stream<NQ, VARIANT, 2>(head, stream, np, base, prio_phase + 2 * st);
-    if (first > 0) walk_stream<NQ, VARIANT, 1>(head, stream, first, base, prio_phase + 2 * st);
+    if (np > 0) TETRIS_STAMP_WALK((walk_stream<NQ, VARIANT, 2>(head, stream, np, base, prio_phase + 2 * st)));
+    if (first > 0) TETRIS_STAMP_WALK((walk_stream<NQ, VARIANT, 1>(head, stream, first, base, prio_phase + 2 * st)));
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): my loads of stage st + 1 have landed
     sink ^= touched;
     __syncthreads();                     // ... and so have everyone's; nobody reads the buffer of stage st - 1 any more
     if (early) issue(st + 2);
-    if (nb - np - first > 0) walk_stream<NQ, VARIANT, 1>(head, stream, nb - np - first, base, prio_phase + 2 * st + 1);
+    if (nb - np - first > 0)
+      TETRIS_STAMP_WALK((walk_stream<NQ, VARIANT, 1>(head, stream, nb - np - first, base, prio_phase + 2 * st + 1)));
     if (late) issue(st + 2);
     o0 = o1; o1 = o2; o2 = o3; o3 = o4;
   }
+  TETRIS_STAMP(5);
 
   // ---- write the outputs -------------------------------------------------------------------------------------
   if (g.N < 0) out[0] = __builtin_bit_cast(float, sink);  // never true: keeps the touching loads alive
@@ -752,6 +825,7 @@ __device__ __forceinline__ void conv3_body(const float* __restrict__ in, float* 
   else store_outputs<NQ, VARIANT>(out + (size_t)slice * out_elems, lane_oc, g, u0, n_base, limg, lrow, lx, lane_ok);
   if (g.fused && drew_last_ticket(tickets, tile_id, wave, g))
     add_slices<NQ>(out, final_out, lane_oc, g, u0, n_base, limg, lrow, lx, lane_ok);
+  TETRIS_STAMP_END();
 }
 
 template <int NQ>
@@ -797,7 +871,9 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
                                           float* __restrict__ final_out, int* __restrict__ tickets, const Geom& g) {
   constexpr int BUF = VARIANT == 8 ? kFlatHalfBufBytes : kFlatBufBytes;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  TETRIS_STAMP_ENTRY();
   touch_kernel_arguments();
+  TETRIS_STAMP_ARGS();
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = uniform(tid >> 6);
@@ -879,8 +955,10 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
       }
     }
   };
+  TETRIS_STAMP(11);
   issue(st0);
   issue(st0 + 1);
+  TETRIS_STAMP(2);
 
   // ---- the wave's streams.  Lane i keeps the stream offset of stage chunk0 + i, so a stage costs no memory access
   // for them (reloaded every 60 stages).
@@ -898,6 +976,7 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
   const int2* stream = entries + o0 + 8;
   Batch head;
   spread_head(head, head_entry);
+  TETRIS_STAMP(3);
   const int* words = reinterpret_cast<const int*>(entries);
   auto touch = [&](int from, int to) {  // pull a stream range into L2: a dword per 128-byte line, 8 KB at most
     const int e = from + lane * 16;
@@ -917,6 +996,7 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
   const int prio_phase = WAVES == 16 ? wave >> 2 : (wave >> 2) * 2;
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): stages st0 and st0 + 1 have landed
   __syncthreads();
+  TETRIS_STAMP(4);
   for (int st = st0; st < st1; ++st) {
     if (st + 3 - chunk0 > 63) {  // the lanes' stream offsets run out: fetch the next 64
       chunk0 = st;
@@ -926,7 +1006,7 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
       __builtin_amdgcn_s_waitcnt(0x0f70);
     }
     const int nb = (o1 - o0) >> 3;
-    if (nb > 0) walk_stream<NQ, VARIANT>(head, stream, nb, lane_base + (st & 1) * BUF, prio_phase + st);
+    if (nb > 0) TETRIS_STAMP_WALK((walk_stream<NQ, VARIANT>(head, stream, nb, lane_base + (st & 1) * BUF, prio_phase + st)));
     o0 = o1;
     o1 = off_at(st + 2);
     if (st + 1 < st1) {
@@ -935,6 +1015,7 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
       issue(st + 2);
     }
   }
+  TETRIS_STAMP(5);
 
   // ---- write the outputs ------------------------------------------------------------------------------------------
   if (g.N < 0) out[0] = __builtin_bit_cast(float, sink);  // never true: keeps the touching loads alive
@@ -971,7 +1052,10 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
       }
     }
   }
-  if (!(g.fused && drew_last_ticket(tickets, tile_id, wave, g))) return;
+  if (!(g.fused && drew_last_ticket(tickets, tile_id, wave, g))) {
+    TETRIS_STAMP_END();
+    return;
+  }
   // This wave adds the slices (see drew_last_ticket): the same quads and channels at the same offsets of every slice.
   const bool fvec = vec && (reinterpret_cast<size_t>(final_out) & 15) == 0;
   const __amdgpu_buffer_rsrc_t frsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -1019,6 +1103,7 @@ __device__ __forceinline__ void flat_body(const float* __restrict__ in, float* _
       }
     }
   }
+  TETRIS_STAMP_END();
 }
 
 template <int NQ>
@@ -1325,3 +1410,17 @@ int launch_conv(const Geom& g0, const float* d_in, float* d_user_out, float* d_s
 }
 
 }  // namespace tetris
+
+#ifdef TETRIS_STAMPS
+// Copies the stamps of the first `n_wg` workgroups of the last launches (16 values each, see TETRIS_STAMP) to the
+// host and clears them.  Only in the library `make stamps` builds.
+extern "C" int tetris_stamps_read(long long* out, int n_wg) {
+  using namespace tetris;
+  if (!out || n_wg < 1 || n_wg > kStampWgs) return fail(TETRIS_EINVAL, "bad argument");
+  TETRIS_HIP(hipDeviceSynchronize());
+  TETRIS_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_stamps), sizeof(long long) * kStampSlots * (size_t)n_wg));
+  std::vector<long long> zero((size_t)kStampSlots * n_wg, 0);
+  TETRIS_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_stamps), zero.data(), sizeof(long long) * zero.size()));
+  return TETRIS_OK;
+}
+#endif

@@ -260,7 +260,8 @@ int make_geom(const tetris_g950* p, int N, int H, int W, int stride, int pad, co
     const long long room = (long long)cu_count() * (g.ver == 3 && four ? 16 : 8);
     const long long waves_total = (long long)g.ugroups * g.kblocks * t.waves;
     if (int rc = choose_csplit(t, waves_total, room, g.stages, &g.csplit)) return rc;
-    if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32))
+    if ((long long)g.ugroups * g.kblocks * g.csplit * g.kblocks * g.csplit >= (1ll << 32) ||
+        (long long)g.stages * (g.csplit + 1) * g.csplit >= (1ll << 32))
       return fail(TETRIS_EINVAL, "grid too large");
     if (g.csplit > 1 && 4ll * g.csplit * N * p->K * g.OH * g.OW > (1ll << 30))
       return fail(TETRIS_EINVAL, "%d slices of this layer's output are more than 1 GiB of partial sums", g.csplit);

@@ -88,6 +88,13 @@ class Tile(C.Structure):
             ", csplit=%d" % self.csplit if self.csplit else "")
 
 
+class LaunchShape(C.Structure):
+    """tetris_launch_shape: how a layer is cut into workgroups for a tile."""
+    _fields_ = [("workgroups", C.c_int32), ("unit_groups", C.c_int32), ("channel_blocks", C.c_int32),
+                ("csplit", C.c_int32), ("stages", C.c_int32), ("lanes_used", C.c_int32), ("kernel", C.c_int32),
+                ("lds_bytes", C.c_int32), ("scratch_bytes", C.c_int64)]
+
+
 _f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
 _i32p_opt = C.c_void_p
 
@@ -125,6 +132,7 @@ _lib.tetris_spconv2d_launch.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C
                                                                                                 C.c_void_p]
 _lib.tetris_g950_prepare.argtypes = [C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile), C.c_void_p]
 _lib.tetris_spconv2d_launch_noalloc.argtypes = _lib.tetris_spconv2d_launch.argtypes
+_lib.tetris_launch_shape_of.argtypes = [C.c_void_p] + [C.c_int] * 5 + [C.POINTER(Tile), C.POINTER(LaunchShape)]
 _lib.tetris_noalloc_scratch_bytes.restype = C.c_size_t
 _lib.tetris_noalloc_scratch_limit.argtypes = [C.c_size_t]
 _lib.tetris_noalloc_scratch_limit.restype = C.c_size_t
@@ -299,6 +307,12 @@ class G950Filter:
         """Makes the launch plan (and a split layer's partial-sum buffer on `stream`) ahead of the first launch."""
         _check(_lib.tetris_g950_prepare(self._h, batch, img_h, img_w, stride, padding,
                                         C.byref(tile) if tile is not None else None, C.c_void_p(stream)))
+
+    def launch_shape(self, batch, img_h, img_w, stride, padding, tile):
+        """How the layer is cut into workgroups for `tile` (tetris_launch_shape_of); nothing is launched."""
+        out = LaunchShape()
+        _check(_lib.tetris_launch_shape_of(self._h, batch, img_h, img_w, stride, padding, C.byref(tile), C.byref(out)))
+        return out
 
     def launch_noalloc(self, d_input, d_output, batch, img_h, img_w, stride, padding, tile=None, stream=0):
         """launch() for callers that cannot allocate: needs prepare() first, uses the library's static scratch array."""
