@@ -289,7 +289,7 @@ def summary_line(full, details):
     rl = full["roofline"]
     line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
                                  "ms_per_step_device", "higher_is_better", "scaling", "vs_baseline", "dtype", "data")}
-    line["metric"] = "effective GFLOP/s (dense-equivalent) of the sparse conv stack"
+    line["metric"] = "effective GFLOP/s (dense-equivalent), sparse conv stack"
     line["config"] = pick(full["config"], ("workload", "suite", "batch", "layers"))
     line["check"] = None if full["check"] is None else pick(full["check"], (
         "ok", "max_rel_err", "tolerance", "all_workloads_ok") + (() if full["check"]["all_workloads_ok"] else ("failed_workloads",)))
@@ -307,7 +307,7 @@ def summary_line(full, details):
                                  "vendor_csr_im2col_ms_per_step"))
     # other workloads: [suite, batch, ms per pass, bound, fraction of the binding roof, smallest layer fraction,
     #                   counter bytes / algorithmic bytes, check ok]
-    line["suites_cols"] = "suite,batch,ms,bound,frac,min_layer_frac,traffic_ratio,check_ok"
+    line["suites_cols"] = "suite,batch,ms,bound,frac,min_layer_frac,traffic_ratio,ok"
     line["suites"] = [[r["suite"], r["batch"], r["ms_per_step_device"], r["bound"].replace("valu_", ""), r["roofline_frac"],
                        r["min_layer_roofline_frac"],
                        round(r["traffic"] / r["algorithmic_bytes_per_launch"], 3) if r.get("traffic") else None,
@@ -413,7 +413,7 @@ def main():
         achieved = fl_sparse / t_step / 1e12
         # the contract's label for the compute roof is "mfma"; the work here is vector fp32 FMA on the VALU, no MFMA
         roofline = {"bound": "mfma", "bound_detail": "valu_fp32",
-                    "note": "VALU fp32 FMA, no MFMA; the peak needs packed fp32 (compiled off here: 78.6 reachable)",
+                    "note": "VALU fp32 FMA, no MFMA; peak needs packed fp32 (off here: 78.6 reachable)",
                     "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / PEAK_FP32_TFLOPS, 4)}
     else:
@@ -474,7 +474,7 @@ def main():
             if t_cpu > budget_s:
                 break
         cpu = {"value": round(done_fl / t_cpu / 1e9, 2), "unit": "GFLOP/s", "cores": threads,
-               "kind": "port", "sample": "first %d of %d %s layers, batch %d, one pass: reference SparseFilter layout (TILE_IC 32, "
+               "kind": "port", "sample": "%d of %d %s layers, batch %d, one pass: reference SparseFilter layout (TILE_IC 32, "
                "Bank-SR + ReorderOutChannel, vec4) decoded by the oracle's HostReorderSpconv2d, OpenMP over (n, oc), %.1f s"
                % (used, len(layers), args.suite, N, t_cpu),
                "pack_s": round(t_cpu_pack, 2),
