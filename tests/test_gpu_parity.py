@@ -744,6 +744,72 @@ def test_slices_of_the_channel_reduction_chosen_by_the_tile(env, case):
     pk.close()
 
 
+def test_launch_shape_query(env):
+    # tetris_launch_shape_of: what the launcher derives from (shape, tile) without launching
+    T, torch, O = env
+    w = sparse_filter(np.random.default_rng(5), 96, 256, 3, 0.9)
+    N, H = 4, 14
+    for t5, cs in [((7, 2, 2, 16, 16), 0), ((7, 2, 2, 16, 16), 1), ((7, 2, 2, 16, 16), 4), ((14, 1, 8, 4, 8), 2)]:
+        tile = T.Tile(*t5, cs)
+        pk = T.G950Filter.for_tile(w, tile)
+        sh = pk.launch_shape(N, H, H, 1, 1, tile)
+        assert sh.stages == -(-256 // t5[4]) and sh.channel_blocks == -(-96 // (t5[2] * t5[3]))
+        assert sh.workgroups == sh.unit_groups * sh.channel_blocks * sh.csplit and 1 <= sh.lanes_used <= 64
+        assert sh.kernel == (3 if t5[3] >= 8 else 2)
+        if cs:
+            assert sh.csplit == cs
+        assert sh.scratch_bytes == (0 if sh.csplit == 1 else 65536 + 4 * sh.csplit * N * 96 * H * H)
+        pk.close()
+    w1 = sparse_filter(np.random.default_rng(6), 64, 128, 1, 0.8)
+    tile = T.Tile(64, 2, 4, 8, 16)
+    pk = T.G950Filter.for_tile(w1, tile)
+    sh = pk.launch_shape(3, 13, 13, 1, 0, tile)
+    assert sh.kernel == 4 and sh.lanes_used == 64 and sh.unit_groups == -(-(-(-(3 * ((169 + 3) // 4)) // 64)) // 2)
+    with pytest.raises(T.TetrisError):
+        pk.launch_shape(3, 13, 13, 1, 0, T.Tile(64, 2, 4, 8, 16, 9))
+    pk.close()
+
+
+def test_raw_launcher_from_several_threads(env):
+    # The raw launchers keep the packs they decode in a small cache that other calls may evict; a call holds the
+    # cache's lock until its launch is issued.  Four threads, each with its own arrays (more sets than the cache
+    # would need to start evicting at 16 is not the point here: concurrent decode + launch is), all results right.
+    T, torch, O = env
+    import threading
+    N, C, H, W, K, ks = 2, 24, 12, 12, 40, 3
+    x = relu_like(np.random.default_rng(70), (N, C, H, W))
+    dx = torch.from_numpy(x).cuda()
+    jobs = []
+    for i in range(20):  # twenty sets of arrays: the cache holds sixteen
+        w = sparse_filter(np.random.default_rng(100 + i), K, C, ks, 0.8)
+        p = O.SpfPack(w, 32, True, True, True, True)
+        jobs.append((w, [torch.from_numpy(np.ascontiguousarray(a)).cuda() for a in p.arrays()],
+                     torch.full((N, K, H, W), float("nan"), device="cuda")))
+    torch.cuda.synchronize()
+    errors = []
+
+    def work(lo):
+        try:
+            for rep in range(3):
+                for w, a, dy in jobs[lo::4]:
+                    T.SparseConv2d(dx.data_ptr(), a[0].data_ptr(), a[1].data_ptr(), a[4].data_ptr(), a[2].data_ptr(),
+                                   a[3].data_ptr(), dy.data_ptr(), N, H, W, C, K, ks, 1, 1, TILE_IC=32, vec_width=4,
+                                   n_entries=a[3].numel())
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for w, a, dy in jobs:
+        assert max_rel_err(dy.cpu().numpy(), O.host_conv2d(x, w, 1, 1, threads=4)) <= TOL
+        T.spf_invalidate(a[3].data_ptr())
+
+
 def test_launches_can_be_captured_in_a_hip_graph(env):
     # After one eager launch per shape (which makes the launch plan and, for a split layer, its scratch buffer) a
     # launch is nothing but kernel launches on the caller's stream, so a chain of layers can be captured once and
