@@ -273,22 +273,18 @@ int view_pack(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_
   if (C <= 0 || K <= 0 || ks <= 0 || ks > kMaxKs || tile_ic <= 0 || (vec != 0 && vec != 1 && vec != 4))
     return fail(TETRIS_EINVAL, "bad filter shape C=%d K=%d ks=%d tile_ic=%d vector width=%d", C, K, ks, tile_ic, vec);
   if (capacity < 0) return fail(TETRIS_EINVAL, "negative entry capacity");
-  SpfView* v = nullptr;
-  for (size_t i = 0; i < g_views.size(); ++i) {
-    SpfView* c = g_views[i];
-    if (c->ptrs[0] == d_offsets && c->ptrs[1] == d_perm && c->ptrs[2] == d_position && c->ptrs[3] == d_values && c->C == C &&
-        c->K == K && c->ks == ks && c->tile_ic == tile_ic && c->vec == vec) {
-      v = c;
-      g_views.erase(g_views.begin() + (long)i);
-      break;
-    }
-  }
+  auto find = [&]() -> SpfView* {  // the view of these addresses and this shape, if there is one
+    for (SpfView* c : g_views)
+      if (c->ptrs[0] == d_offsets && c->ptrs[1] == d_perm && c->ptrs[2] == d_position && c->ptrs[3] == d_values &&
+          c->C == C && c->K == K && c->ks == ks && c->tile_ic == tile_ic && c->vec == vec)
+        return c;
+    return nullptr;
+  };
+  SpfView* v = find();
   const bool trusted = v && v->d_filter && (options() & TETRIS_OPT_TRUST_SPF_ARRAYS);
   unsigned long long hash = v ? v->hash : 0;
   int rc = TETRIS_OK;
   if (!trusted) {
-    if (v) g_views.push_back(v);  // stays registered whatever the checks below say
-    v = nullptr;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
       return fail(TETRIS_EINVAL, "this entry point reads the arrays back (a synchronisation): it cannot be captured; "
@@ -309,16 +305,8 @@ int view_pack(const int32_t* d_offsets, const int32_t* d_perm, const int32_t* d_
                          &hash);
     if (rc) return rc;
     hash ^= 0x5bd1e995ull * (unsigned long long)(C * 131 + ks) + (unsigned long long)tile_ic * 7919ull + (unsigned)vec;
-    for (size_t i = 0; i < g_views.size(); ++i) {
-      SpfView* c = g_views[i];
-      if (c->ptrs[0] == d_offsets && c->ptrs[1] == d_perm && c->ptrs[2] == d_position && c->ptrs[3] == d_values &&
-          c->C == C && c->K == K && c->ks == ks && c->tile_ic == tile_ic && c->vec == vec) {
-        v = c;
-        g_views.erase(g_views.begin() + (long)i);
-        break;
-      }
-    }
   }
+  if (v) g_views.erase(std::find(g_views.begin(), g_views.end(), v));  // moves to the most-recently-used end below
   if (!v) {
     v = new SpfView;
     v->ptrs[0] = d_offsets; v->ptrs[1] = d_perm; v->ptrs[2] = d_position; v->ptrs[3] = d_values;
