@@ -112,3 +112,30 @@ def test_choose_refuses_counter_files_that_do_not_match_the_shortlist(tmp_path):
                         "--write", str(tmp_path / "write"), "--out", str(tmp_path / "t.inc")], capture_output=True, text=True,
                        env=env, timeout=120)
     assert r.returncode != 0 and "conv launches" in r.stderr
+
+
+def test_table_rows_with_and_without_csplit(tmp_path):
+    """A table row's tile has five numbers, or six when it fixes csplit: the tuner's writer and reader agree on both,
+    and the library's own loader (tetris_tile_table_load) reads what the tuner writes."""
+    sys.path.insert(0, PKG)
+    import tetris_amd as T
+    from tetris_amd import tune
+
+    rows = [((2, 13, 13, 512, 256, 1, 1, 0), (64, 1, 1, 16, 64, 4), "with csplit"),
+            ((16, 56, 56, 256, 256, 3, 1, 1), (14, 2, 8, 16, 16), "rule")]
+    path = tmp_path / "t.inc"
+    tune.write_table(str(path), rows)
+    pat = re.compile(tune.ROW + r",\s*// (.*)")
+    got = []
+    for ln in open(path):
+        m = pat.match(ln)
+        if m:
+            g = m.groups()
+            got.append((tuple(int(x) for x in g[:8]), tune.row_tile(g), g[14]))
+    assert got == rows
+    n = T.tile_table_load(str(path))
+    assert n == 2
+    t = T.tile_select(2, 13, 13, 512, 256, 1, 1, 0)
+    assert t.as_list() == [64, 1, 1, 16, 64, 4] and "csplit=4" in repr(t)
+    t = T.tile_select(16, 56, 56, 256, 256, 3, 1, 1)
+    assert t.as_list() == [14, 2, 8, 16, 16] and t.csplit == 0
