@@ -12,10 +12,11 @@ batch, first stage landed and barrier, stage loop (with the share of it that the
 spent inside the walk), output stores issued, stores acknowledged -- plus when the last workgroup entered and the
 device span of the conv kernel (first entry to last exit; the rest of the launch time is the gap before the kernel
 and, for a split layer, the kernel that adds the slices).
---worst N picks the N layers furthest below their roof (timed first with the same build).
+--worst N lists only the N layers furthest below their roof (the waterfall's `all` row stays over every layer).
 --waterfall prints, per layer and for the whole selection, the chain of factors from the vector units' rate to the
 measured time: FMA-only time at the measured shader clock -> x loop (cycles per entry over FMA cycles per entry) ->
-x lanes (lanes that own pixels) -> x workgroup slots filled -> x walking share -> x stage loop's share of the kernel
+x lanes (lanes that own pixels) -> x workgroup slots filled -> x share of the stage loop a wave spends walking, mean
+over the waves (a SIMD works at the loop's rate while its waves walk) -> x stage loop's share of the kernel
 -> x kernel's share of the launch.  The stamped build reads the clock around every walk call, which costs about a
 tenth of the stage loop's time: its launch times are that much longer than the product build's, the shares hold.
 """
@@ -29,9 +30,10 @@ import tetris_amd as T
 from tetris_amd import workloads as W
 
 SLOTS, MAX_WGS = 16, 8192
-# cycles of a SIMD per entry at four / two waves per SIMD, measured on the loop alone (quads -> cycles); an entry's FMAs
-# alone take 16 cycles per quad
+# time of a SIMD per entry at four / two waves per SIMD, measured on the loop alone (quads -> periods of the nominal
+# 2.4 GHz clock, the unit the loop's micro-benchmark reports); an entry's FMAs alone take 16 shader cycles per quad
 LOOP_CYCLES = {True: {1: 26.2, 2: 43.5}, False: {1: 30.0, 2: 50.0, 4: 85.2}}
+NOMINAL_MHZ = 2400.0
 
 
 def read_stamps():
@@ -58,8 +60,9 @@ def breakdown(torch, L, batch, cold):
         torch.cuda.synchronize()
     pk.launch(*args)
     s = read_stamps().astype(np.float64)
+    nnz = pk.host_arrays()["nnz"]
     pk.close()
-    mhz = 100.0 * float((s[:, 7] - s[:, 0]).sum()) / max(float((s[:, 10] - s[:, 9]).sum()), 1.0)  # shader clock / 100 MHz
+    mhz = 100.0 * float((s[:, 7] - s[:, 0]).sum()) / max(float((s[:, 10] - s[:, 9]).sum()), 1.0)  # shader clock in MHz (cycles per 100 MHz tick x 100)
     us = lambda a: float(np.mean(a)) / mhz  # noqa: E731
     loop = s[:, 5] - s[:, 4]
     four = tile.waves == 16 or (tile.waves == 8 and tile.oc_per_wave * 4 * tile.quads <= 64 and tile.quads <= 2)
@@ -67,6 +70,14 @@ def breakdown(torch, L, batch, cold):
     slots = 256 * (1 if tile.waves == 16 or (tile.waves == 8 and not four) else 2)
     rounds = -(-shape.workgroups // slots)
     wk = W.work(L, batch)
+    lanes = shape.lanes_used / 64.0
+    if tile.lanes_w == 64:  # flat tile: 64 consecutive quads of the batch per unit, the last unit of the batch part empty
+        quads = batch * -(-(oh * ow) // 4)
+        lanes = quads / (64.0 * -(-quads // 64))
+    # shader cycles per entry: the micro-benchmark's time per entry at the shader clock measured here (the FMA rate the
+    # box sustains under load corresponds to this clock, not to the nominal one)
+    nominal = LOOP_CYCLES[four].get(tile.quads)
+    loop_cycles = nominal * mhz / NOMINAL_MHZ if nominal else 16.0 * tile.quads
     return {"layer": L.name, "tile": tile.as_list(), "wgs": len(s), "launch_us": ms * 1e3, "csplit": shape.csplit,
             "args": us(s[:, 1] - s[:, 0]), "issued": us(s[:, 2] - s[:, 1]), "head": us(s[:, 3] - s[:, 2]),
             "landed": us(s[:, 4] - s[:, 3]), "loop": us(loop),
@@ -75,37 +86,42 @@ def breakdown(torch, L, batch, cold):
             "stores": us(s[:, 6] - s[:, 5]), "acked": us(s[:, 7] - s[:, 6]),
             "last_entry": float(s[:, 9].max() - s[:, 9].min()) / 100.0, "span": float(s[:, 10].max() - s[:, 9].min()) / 100.0,
             "kernel": us(s[:, 7] - s[:, 0]), "mhz": mhz, "roof_us": wk["t_roof"] * 1e6, "flops": wk["flops_sparse"],
-            "lanes": shape.lanes_used / 64.0, "fill": shape.workgroups / float(rounds * slots), "rounds": rounds,
-            "loop_eff": 16.0 * tile.quads / LOOP_CYCLES[four].get(tile.quads, 16.0 * tile.quads)}
+            "lanes": lanes, "fill": shape.workgroups / float(rounds * slots), "rounds": rounds,
+            "loop_eff": 16.0 * tile.quads / loop_cycles, "loop_cycles": loop_cycles,
+            # every unit group walks every non-zero once; a SIMD holds waves / 4 of the workgroup's waves (times two
+            # workgroups where two fit a CU), and while they all walk, the SIMD's cycles per entry are one wave's
+            # cycles inside the walk over its entries, divided by the waves that share the SIMD
+            "seen_cycles": float(s[:, 13].sum()) / (tile.waves / 4.0 * (slots // 256)) / max(nnz * shape.unit_groups, 1)}
 
 
-def waterfall(rows):
-    """Per layer and in total: the time the FMAs alone would take on 256 CUs x 4 SIMDs x 16 lanes at the measured clock,
-    and the factors that lead from there to the measured launch time."""
-    print("\n| layer | FMA-only us | loop | lanes | slots filled | busiest wave walking | stage loop / kernel | kernel / "
-          "launch | product | measured us | FMA-only / measured |")
-    print("|" + "---|" * 11)
+def waterfall(rows, shown):
+    """Per layer (those of `shown`) and in total (all of `rows`): the time the FMAs alone would take on 256 CUs x 4 SIMDs
+    x 16 lanes at the measured clock, and the factors that lead from there to the measured launch time."""
+    print("\n| layer | FMA-only us | loop | lanes | slots filled | waves walking | stage loop / kernel | kernel / "
+          "launch | product | measured us | FMA-only / measured | SIMD cycles per entry: in the kernel (loop alone) |")
+    print("|" + "---|" * 12)
     tot = dict(ideal=0.0, meas=0.0)
-    acc = {k: 0.0 for k in ("loop_eff", "lanes", "fill", "walk_max", "loop_share", "kern_share")}
+    acc = {k: 0.0 for k in ("loop_eff", "lanes", "fill", "walk_mean", "loop_share", "kern_share")}
     for r in rows:
         ideal = r["flops"] / 2.0 / (256 * 4 * 16) / r["mhz"]  # FMAs / (lanes of the GPU) / MHz = microseconds
         loop_share = r["loop"] / r["kernel"]
         # one round of workgroups: the launch is a workgroup's life plus what lies around the kernel; several rounds: a
         # CU starts its next workgroup as one ends, the launch is the sum of lives (the idle slots are under "filled")
         kern_share = min(1.0, r["rounds"] * r["kernel"] / r["launch_us"])
-        prod = r["loop_eff"] * r["lanes"] * r["fill"] * r["walk_max"] * loop_share * kern_share
-        print("| %s | %.1f | %.2f | %.2f | %.2f | %.2f | %.2f | %.2f | %.3f | %.1f | %.3f |" % (
-            r["layer"], ideal, r["loop_eff"], r["lanes"], r["fill"], r["walk_max"], loop_share, kern_share, prod,
-            r["launch_us"], ideal / r["launch_us"]))
+        prod = r["loop_eff"] * r["lanes"] * r["fill"] * r["walk_mean"] * loop_share * kern_share
+        if any(r is x for x in shown):
+            print("| %s | %.1f | %.2f | %.2f | %.2f | %.2f | %.2f | %.2f | %.3f | %.1f | %.3f | %.1f (%.1f) |" % (
+                r["layer"], ideal, r["loop_eff"], r["lanes"], r["fill"], r["walk_mean"], loop_share, kern_share, prod,
+                r["launch_us"], ideal / r["launch_us"], r["seen_cycles"], r["loop_cycles"]))
         tot["ideal"] += ideal
         tot["meas"] += r["launch_us"]
-        for k, v in (("loop_eff", r["loop_eff"]), ("lanes", r["lanes"]), ("fill", r["fill"]), ("walk_max", r["walk_max"]),
+        for k, v in (("loop_eff", r["loop_eff"]), ("lanes", r["lanes"]), ("fill", r["fill"]), ("walk_mean", r["walk_mean"]),
                      ("loop_share", loop_share), ("kern_share", kern_share)):
             acc[k] += v * r["launch_us"]  # weighted by where the time is spent
     w = {k: v / tot["meas"] for k, v in acc.items()}
-    print("| all (time-weighted) | %.1f | %.2f | %.2f | %.2f | %.2f | %.2f | %.2f | %.3f | %.1f | %.3f |" % (
-        tot["ideal"], w["loop_eff"], w["lanes"], w["fill"], w["walk_max"], w["loop_share"], w["kern_share"],
-        w["loop_eff"] * w["lanes"] * w["fill"] * w["walk_max"] * w["loop_share"] * w["kern_share"], tot["meas"],
+    print("| all (time-weighted) | %.1f | %.2f | %.2f | %.2f | %.2f | %.2f | %.2f | %.3f | %.1f | %.3f | |" % (
+        tot["ideal"], w["loop_eff"], w["lanes"], w["fill"], w["walk_mean"], w["loop_share"], w["kern_share"],
+        w["loop_eff"] * w["lanes"] * w["fill"] * w["walk_mean"] * w["loop_share"] * w["kern_share"], tot["meas"],
         tot["ideal"] / tot["meas"]))
 
 
@@ -114,7 +130,7 @@ def main():
     ap.add_argument("--suite", default="vgg19")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--layers", nargs="*", help="layer names (substrings); default: all")
-    ap.add_argument("--worst", type=int, default=0, help="only the N layers furthest below their roof")
+    ap.add_argument("--worst", type=int, default=0, help="list only the N layers furthest below their roof")
     ap.add_argument("--cold", action="store_true", help="evict the caches before the stamped launch")
     ap.add_argument("--waterfall", action="store_true", help="also print the chain of factors from the FMA rate to the time")
     args = ap.parse_args()
@@ -125,8 +141,7 @@ def main():
                  "TETRIS_SPCONV2D_LIB to build_stamps/libtetris_spconv2d.so" % T.LIB_PATH)
     layers = [L for L in W.SUITES[args.suite]() if not args.layers or any(n in L.name for n in args.layers)]
     rows = [breakdown(torch, L, args.batch, args.cold) for L in layers]
-    if args.worst:
-        rows = sorted(rows, key=lambda r: r["roof_us"] / r["launch_us"])[:args.worst]
+    shown = sorted(rows, key=lambda r: r["roof_us"] / r["launch_us"])[:args.worst] if args.worst else rows
     print("%s at batch %d%s; shader clock %.0f MHz; microseconds, mean over a layer's workgroups\n" %
           (args.suite, args.batch, ", caches evicted before the stamped launch" if args.cold else "",
            float(np.mean([r["mhz"] for r in rows]))))
@@ -134,13 +149,13 @@ def main():
           "stage issued | offsets + first batch | first stage landed + barrier | stage loop (walking: busiest wave, mean "
           "wave) | stores issued | stores acknowledged | last workgroup enters after | conv kernel span |")
     print("|" + "---|" * 14)
-    for r in rows:
+    for r in shown:
         print("| %s | %s | %d (%d) | %.1f | %.3f | %.2f | %.2f | %.2f | %.2f | %.1f (%.2f, %.2f) | %.2f | %.2f | %.2f | %.1f |" % (
             r["layer"], r["tile"], r["wgs"], r["csplit"], r["launch_us"], r["roof_us"] / r["launch_us"], r["args"],
             r["issued"], r["head"], r["landed"], r["loop"], r["walk_max"], r["walk_mean"], r["stores"], r["acked"],
             r["last_entry"], r["span"]))
     if args.waterfall:
-        waterfall(rows)
+        waterfall(rows, shown)
 
 
 if __name__ == "__main__":
