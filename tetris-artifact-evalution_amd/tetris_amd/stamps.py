@@ -15,10 +15,11 @@ and, for a split layer, the kernel that adds the slices).
 --worst N lists only the N layers furthest below their roof (the waterfall's `all` row stays over every layer).
 --waterfall prints, per layer and for the whole selection, the chain of factors from the vector units' rate to the
 measured time: FMA-only time at the measured shader clock -> x loop (cycles per entry over FMA cycles per entry) ->
-x lanes (lanes that own pixels) -> x workgroup slots filled -> x share of the stage loop a wave spends walking, mean
-over the waves (a SIMD works at the loop's rate while its waves walk) -> x stage loop's share of the kernel
--> x kernel's share of the launch.  The stamped build reads the clock around every walk call, which costs about a
-tenth of the stage loop's time: its launch times are that much longer than the product build's, the shares hold.
+x lanes (lanes that own pixels) -> x workgroup slots filled -> x share of the stage loop the busiest wave spends
+walking (a SIMD works at the loop's rate while that wave walks) -> x stage loop's share of the kernel
+-> x kernel's share of the launch.  The stamped build reads the clock around every walk call, which makes a pass
+some 2 % longer than the product build's.  Every layer is launched for about 30 ms before it is timed, so that the
+shader clock is where a whole pass holds it.
 """
 import argparse
 import ctypes as C
@@ -30,10 +31,10 @@ import tetris_amd as T
 from tetris_amd import workloads as W
 
 SLOTS, MAX_WGS = 16, 8192
-# time of a SIMD per entry at four / two waves per SIMD, measured on the loop alone (quads -> periods of the nominal
-# 2.4 GHz clock, the unit the loop's micro-benchmark reports); an entry's FMAs alone take 16 shader cycles per quad
+# shader cycles of a SIMD per entry at four / two waves per SIMD, measured on the loop alone in a kernel that runs long
+# enough for the clock to settle near the nominal 2.4 GHz its time is divided by (quads -> cycles); an entry's FMAs
+# alone take 16 cycles per quad
 LOOP_CYCLES = {True: {1: 26.2, 2: 43.5}, False: {1: 30.0, 2: 50.0, 4: 85.2}}
-NOMINAL_MHZ = 2400.0
 
 
 def read_stamps():
@@ -53,8 +54,12 @@ def breakdown(torch, L, batch, cold):
     dx = torch.from_numpy(x).cuda()
     dy = torch.empty((batch, L.K, oh, ow), device="cuda")
     args = (dx.data_ptr(), dy.data_ptr(), batch, L.H, L.W, L.stride, L.pad, tile)
-    ms = pk.time(*args, warm=5, repeat=20)
-    read_stamps()  # clears what the timed launches left
+    # The shader clock idles at about 2.1 GHz and takes 10-25 ms of unbroken work to reach the 2.3-2.4 GHz that a
+    # whole pass runs at: launch some 30 ms' worth before the timed launches; the stamped launch follows at once (the
+    # clock does not fall back during the fraction of a millisecond that clearing the stamps takes).
+    ms = pk.time(*args, warm=2, repeat=5)
+    ms = pk.time(*args, warm=max(5, min(3000, int(30.0 / ms))), repeat=20)
+    read_stamps()  # clears what the timed launches left (the walk's cycle counts add up from launch to launch)
     if cold:
         torch.empty(128 << 20, dtype=torch.float32, device="cuda").fill_(1.0)  # 512 MiB: evicts the caches
         torch.cuda.synchronize()
@@ -74,10 +79,10 @@ def breakdown(torch, L, batch, cold):
     if tile.lanes_w == 64:  # flat tile: 64 consecutive quads of the batch per unit, the last unit of the batch part empty
         quads = batch * -(-(oh * ow) // 4)
         lanes = quads / (64.0 * -(-quads // 64))
-    # shader cycles per entry: the micro-benchmark's time per entry at the shader clock measured here (the FMA rate the
-    # box sustains under load corresponds to this clock, not to the nominal one)
-    nominal = LOOP_CYCLES[four].get(tile.quads)
-    loop_cycles = nominal * mhz / NOMINAL_MHZ if nominal else 16.0 * tile.quads
+    loop_cycles = LOOP_CYCLES[four].get(tile.quads, 16.0 * tile.quads)
+    # entries a SIMD walks in the stage loop: a workgroup's share of the non-zeros, a quarter of it per SIMD, times the
+    # workgroups that share the CU
+    simd_entries = nnz / float(shape.channel_blocks * shape.csplit) / 4.0 * (slots // 256)
     return {"layer": L.name, "tile": tile.as_list(), "wgs": len(s), "launch_us": ms * 1e3, "csplit": shape.csplit,
             "args": us(s[:, 1] - s[:, 0]), "issued": us(s[:, 2] - s[:, 1]), "head": us(s[:, 3] - s[:, 2]),
             "landed": us(s[:, 4] - s[:, 3]), "loop": us(loop),
@@ -88,40 +93,38 @@ def breakdown(torch, L, batch, cold):
             "kernel": us(s[:, 7] - s[:, 0]), "mhz": mhz, "roof_us": wk["t_roof"] * 1e6, "flops": wk["flops_sparse"],
             "lanes": lanes, "fill": shape.workgroups / float(rounds * slots), "rounds": rounds,
             "loop_eff": 16.0 * tile.quads / loop_cycles, "loop_cycles": loop_cycles,
-            # every unit group walks every non-zero once; a SIMD holds waves / 4 of the workgroup's waves (times two
-            # workgroups where two fit a CU), and while they all walk, the SIMD's cycles per entry are one wave's
-            # cycles inside the walk over its entries, divided by the waves that share the SIMD
-            "seen_cycles": float(s[:, 13].sum()) / (tile.waves / 4.0 * (slots // 256)) / max(nnz * shape.unit_groups, 1)}
+            # what the SIMD spends per entry if it is busy whenever the busiest wave walks: to set beside loop_cycles
+            "seen_cycles": float(np.mean(loop)) * float(s[:, 12].sum() / max(loop.sum(), 1.0)) / max(simd_entries, 1.0)}
 
 
 def waterfall(rows, shown):
     """Per layer (those of `shown`) and in total (all of `rows`): the time the FMAs alone would take on 256 CUs x 4 SIMDs
     x 16 lanes at the measured clock, and the factors that lead from there to the measured launch time."""
-    print("\n| layer | FMA-only us | loop | lanes | slots filled | waves walking | stage loop / kernel | kernel / "
-          "launch | product | measured us | FMA-only / measured | SIMD cycles per entry: in the kernel (loop alone) |")
+    print("\n| layer | FMA-only us | loop | lanes | slots filled | busiest wave walking | stage loop / kernel | kernel / "
+          "launch | product | measured us | FMA-only / measured | SIMD cycles per entry while the busiest wave walks (loop alone) |")
     print("|" + "---|" * 12)
     tot = dict(ideal=0.0, meas=0.0)
-    acc = {k: 0.0 for k in ("loop_eff", "lanes", "fill", "walk_mean", "loop_share", "kern_share")}
+    acc = {k: 0.0 for k in ("loop_eff", "lanes", "fill", "walk_max", "loop_share", "kern_share")}
     for r in rows:
         ideal = r["flops"] / 2.0 / (256 * 4 * 16) / r["mhz"]  # FMAs / (lanes of the GPU) / MHz = microseconds
         loop_share = r["loop"] / r["kernel"]
         # one round of workgroups: the launch is a workgroup's life plus what lies around the kernel; several rounds: a
         # CU starts its next workgroup as one ends, the launch is the sum of lives (the idle slots are under "filled")
         kern_share = min(1.0, r["rounds"] * r["kernel"] / r["launch_us"])
-        prod = r["loop_eff"] * r["lanes"] * r["fill"] * r["walk_mean"] * loop_share * kern_share
+        prod = r["loop_eff"] * r["lanes"] * r["fill"] * r["walk_max"] * loop_share * kern_share
         if any(r is x for x in shown):
             print("| %s | %.1f | %.2f | %.2f | %.2f | %.2f | %.2f | %.2f | %.3f | %.1f | %.3f | %.1f (%.1f) |" % (
-                r["layer"], ideal, r["loop_eff"], r["lanes"], r["fill"], r["walk_mean"], loop_share, kern_share, prod,
+                r["layer"], ideal, r["loop_eff"], r["lanes"], r["fill"], r["walk_max"], loop_share, kern_share, prod,
                 r["launch_us"], ideal / r["launch_us"], r["seen_cycles"], r["loop_cycles"]))
         tot["ideal"] += ideal
         tot["meas"] += r["launch_us"]
-        for k, v in (("loop_eff", r["loop_eff"]), ("lanes", r["lanes"]), ("fill", r["fill"]), ("walk_mean", r["walk_mean"]),
+        for k, v in (("loop_eff", r["loop_eff"]), ("lanes", r["lanes"]), ("fill", r["fill"]), ("walk_max", r["walk_max"]),
                      ("loop_share", loop_share), ("kern_share", kern_share)):
             acc[k] += v * r["launch_us"]  # weighted by where the time is spent
     w = {k: v / tot["meas"] for k, v in acc.items()}
     print("| all (time-weighted) | %.1f | %.2f | %.2f | %.2f | %.2f | %.2f | %.2f | %.3f | %.1f | %.3f | |" % (
-        tot["ideal"], w["loop_eff"], w["lanes"], w["fill"], w["walk_mean"], w["loop_share"], w["kern_share"],
-        w["loop_eff"] * w["lanes"] * w["fill"] * w["walk_mean"] * w["loop_share"] * w["kern_share"], tot["meas"],
+        tot["ideal"], w["loop_eff"], w["lanes"], w["fill"], w["walk_max"], w["loop_share"], w["kern_share"],
+        w["loop_eff"] * w["lanes"] * w["fill"] * w["walk_max"] * w["loop_share"] * w["kern_share"], tot["meas"],
         tot["ideal"] / tot["meas"]))
 
 
