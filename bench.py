@@ -9,9 +9,11 @@ kernel, a CPU baseline measured on this box's cores, and one row of scalars for 
 metric (the single layer at batch 1, VGG19 at batch 1/4/8, ResNet-50, MobileNet and YOLOv3 at batch 16).
 Per-layer microseconds and roofline fractions of every workload go to the file --details names.  Every layer
 of every timed workload is compared with the CPU oracle on the whole batch; a mismatch beyond 1e-4 makes
-the exit status non-zero.
+the exit status non-zero.  Before the W warm-up steps of a workload, untimed passes of the same workload run for
+--settle-ms (30 ms): the shader clock idles near 2.1 GHz and needs 10-25 ms of unbroken work to reach the 2.3-2.4 GHz
+it holds under load, which short workloads would otherwise be timed without (`settle_ms` in the output).
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--suite vgg19|resnet50|mobilenet|yolov3|single]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--settle-ms 30] [--suite vgg19|resnet50|mobilenet|yolov3|single]
                   [--batch N] [--no-cpu] [--no-check] [--no-suites] [--details FILE]
 """
 import argparse
@@ -99,6 +101,17 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
         for L, pk, tile, x, y in zip(layers, packs, tiles, xs, ys):
             pk.launch(x.data_ptr(), y.data_ptr(), N, L.H, L.W, L.stride, L.pad, tile)
 
+    def settle():
+        """The shader clock idles near 2.1 GHz and needs 10-25 ms of unbroken work to reach the 2.3-2.4 GHz it holds
+        under load: untimed passes for --settle-ms before anything is timed, so that short workloads are not measured
+        on the ramp (a tenth in time)."""
+        t_s = time.perf_counter()
+        while (time.perf_counter() - t_s) * 1e3 < args.settle_ms:
+            for _ in range(4):
+                step()
+            torch.cuda.synchronize()
+
+    settle()
     for _ in range(warmup):
         step()
     # The launches go to the null stream, which is torch's current stream here, so torch's events bracket them.
@@ -139,6 +152,8 @@ def run_workload(T, W, torch, np, O, args, suite, N, steps, warmup, layer_repeat
     # per-layer table: events on the launch stream around back-to-back launches (reference protocol,
     # Tetris/spconv2d.cc:44-68, with fewer repetitions so the default run stays short)
     table, t_layers = [], 0.0
+    if layer_repeat > 0:
+        settle()  # the check above left the GPU idle
     for L, pk, tile, x, y, wk in zip(layers, packs, tiles, xs, ys, works):
         if layer_repeat <= 0:
             break
@@ -212,6 +227,10 @@ def run_chain(T, W, torch, np, O, args, N, steps, warmup):
             x = a
 
     def timed(fn):
+        t_s = time.perf_counter()  # untimed passes until the shader clock has settled (see run_workload)
+        while (time.perf_counter() - t_s) * 1e3 < args.settle_ms:
+            fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -287,7 +306,7 @@ def summary_line(full, details):
         return {k: d[k] for k in keys if d is not None and k in d}
 
     rl = full["roofline"]
-    line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+    line = {k: full[k] for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "settle_ms", "ms_per_step",
                                  "ms_per_step_device", "higher_is_better", "scaling", "vs_baseline", "dtype", "data")}
     line["metric"] = "effective GFLOP/s (dense-equivalent), sparse conv stack"
     line["config"] = pick(full["config"], ("workload", "suite", "batch", "layers"))
@@ -326,6 +345,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--settle-ms", type=float, default=30.0, help="untimed passes for this long before the warm-up steps "
+                    "of every timed workload, so that the shader clock is where it stays under load (0: none)")
     ap.add_argument("--suite", default="vgg19")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--masks", metavar="NPZ", help="run the layers of a pruned network instead of --suite: a mask file "
@@ -562,6 +583,8 @@ def main():
         "check": dict(check or {}, all_workloads_ok=not failed, failed_workloads=failed) if not args.no_check else None,
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "ms_per_step_device": round(ms_per_step_dev, 4),
+        # untimed passes of the same workload before the W warm-up steps, until the shader clock has settled
+        "settle_ms": args.settle_ms,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s-shaped sparse conv stack, %d layers, batch %d, fp32 NCHW, seeded masks"
                    % (args.suite, len(layers), N), "suite": args.suite, "batch": N, "layers": len(layers),

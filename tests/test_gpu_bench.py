@@ -71,7 +71,7 @@ def test_summary_line_stays_short():
                "min_layer_roofline_frac": 0.0432, "traffic": 1049550000.0, "algorithmic_bytes_per_launch": 689550000.0,
                "check": {"ok": True}, "layers": [{"layer": "x" * 20, "us": 1.0}] * 75} for s, b in bench.OTHER_WORKLOADS]
     full = {"metric": "m", "value": 298123.4, "unit": "GFLOP/s", "n_gpus": 1, "steps": 20, "warmup": 5,
-            "ms_per_step": 2.0912, "ms_per_step_device": 2.0907, "higher_is_better": True, "scaling": "weak",
+            "settle_ms": 30.0, "ms_per_step": 2.0912, "ms_per_step_device": 2.0907, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": "w" * 100, "suite": "vgg19", "batch": 16, "layers": 16, "tensor_seed": "t" * 200},
             "check": {"ok": True, "layers_checked": 16, "max_rel_err": 3.8123456789e-05, "tolerance": 1e-4,
